@@ -1,0 +1,79 @@
+"""Encoder-layer glue and the memory-bound epilogues, restated in PyTorch-CPU fp32.
+
+Test infrastructure (see oracle/__init__.py).  Follows
+  * layers/kernels/add_bias_and_transpose.cu:118-195   bias + Q scale + head split
+  * layers/kernels/add_bias_and_layernorm.cu:191-266   LN(out + bias + residual) * gamma + beta
+  * layers/kernels/add_bias_act.cu:41-48, :86-105      tanh-form GELU of (out + bias)
+  * layers/multi_headed_attention.cpp:154-216, layers/bert_intermediate.cpp:7-29,
+    layers/bert_output.cpp:7-44                        call order and buffer roles
+  * python/modeling_big_bird.py:1318-1329, :1424-1451, :1564-1567  the same glue in the
+    reference's oracle (SelfOutput, Intermediate, Output, feed_forward_chunk)
+Weights are stored `[in, out]` as the reference stores them
+(python/modeling_bert.py:84-91, :107-113, :137-163); the fused QKV weight is Q|K|V.
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from . import attention
+
+GELU_C0 = 0.7978845608028654     # sqrt(2/pi), layers/kernels/add_bias_act.cu:44
+GELU_C1 = 0.044715
+
+
+def bias_residual_layernorm(x, residual, bias, gamma, beta, eps):
+    h = x.float() + bias.float() + residual.float()
+    return F.layer_norm(h, (h.shape[-1],), gamma.float(), beta.float(), eps)
+
+
+def bias_gelu(x, bias):
+    return F.gelu(x.float() + bias.float(), approximate="tanh")
+
+
+def qkv_bias_split(qkv, bias, heads, scale=None):
+    """[T, 3D] -> q, k, v [T, H, d] with the bias added and q multiplied by `scale`
+    (default 1/sqrt(d), layers/kernels/add_bias_and_transpose.cu:183, :214)."""
+    t, d3 = qkv.shape
+    dm = d3 // 3
+    d = dm // heads
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    x = qkv.float() + bias.float()
+    q = (x[:, :dm] * scale).view(t, heads, d)
+    k = x[:, dm:2 * dm].view(t, heads, d)
+    v = x[:, 2 * dm:].view(t, heads, d)
+    return q, k, v
+
+
+def attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block=64):
+    """QKV projection -> split -> block-sparse attention -> out-proj -> bias+residual+LN
+    (layers/multi_headed_attention.cpp:154-216)."""
+    qkv = hidden.float() @ w["qkv_weight"].float()
+    q, k, v = qkv_bias_split(qkv, w["qkv_bias"], heads)
+    ctx = attention.csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block, scale=1.0)
+    proj = ctx @ w["attn_out_weight"].float()
+    return bias_residual_layernorm(proj, hidden, w["attn_out_bias"], w["attn_ln_weight"],
+                                   w["attn_ln_bias"], eps)
+
+
+def encoder_layer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps=1e-5, block=64):
+    """One layer: attention sub-layer, FFN up + GELU, FFN down + bias+residual+LN with the
+    attention output as the residual (python/modeling_bert.py:172-210)."""
+    attn = attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block)
+    inter = bias_gelu(attn @ w["inter_weight"].float(), w["inter_bias"])
+    out = inter @ w["out_weight"].float()
+    return bias_residual_layernorm(out, attn, w["out_bias"], w["out_ln_weight"], w["out_ln_bias"], eps)
+
+
+def random_layer_weights(hidden, ffn, generator, std=0.02, dtype=torch.float32):
+    """N(0, 0.02) weights and biases, gamma = 1, beta = 0."""
+    def n(*shape):
+        return (torch.randn(*shape, generator=generator) * std).to(dtype)
+    return {
+        "qkv_weight": n(hidden, 3 * hidden), "qkv_bias": n(3 * hidden),
+        "attn_out_weight": n(hidden, hidden), "attn_out_bias": n(hidden),
+        "attn_ln_weight": torch.ones(hidden, dtype=dtype), "attn_ln_bias": torch.zeros(hidden, dtype=dtype),
+        "inter_weight": n(hidden, ffn), "inter_bias": n(ffn),
+        "out_weight": n(ffn, hidden), "out_bias": n(hidden),
+        "out_ln_weight": torch.ones(hidden, dtype=dtype), "out_ln_bias": torch.zeros(hidden, dtype=dtype),
+    }

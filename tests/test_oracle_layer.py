@@ -1,0 +1,54 @@
+"""Layer glue and epilogues of the oracle against library routines."""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from oracle import layer as ol
+from oracle import metadata as md
+
+
+def test_gelu_constants_and_library():
+    x = torch.linspace(-6, 6, 1001)
+    b = torch.zeros(1001)
+    hand = 0.5 * x * (1 + torch.tanh(ol.GELU_C0 * (x + ol.GELU_C1 * x ** 3)))
+    assert (ol.bias_gelu(x, b) - hand).abs().max().item() < 1e-6
+    assert abs(ol.GELU_C0 - math.sqrt(2 / math.pi)) < 1e-12
+
+
+def test_layernorm_by_hand():
+    torch.manual_seed(0)
+    x, r = torch.randn(5, 768), torch.randn(5, 768)
+    b, g, be = torch.randn(768), torch.randn(768), torch.randn(768)
+    h = (x + b + r).double()
+    mu = h.mean(-1, keepdim=True)
+    var = ((h - mu) ** 2).mean(-1, keepdim=True)
+    want = (h - mu) / torch.sqrt(var + 1e-5) * g.double() + be.double()
+    assert (ol.bias_residual_layernorm(x, r, b, g, be, 1e-5).double() - want).abs().max().item() < 1e-5
+
+
+def test_qkv_split_is_reshape_permute():
+    torch.manual_seed(0)
+    qkv, bias = torch.randn(128, 3 * 768), torch.randn(3 * 768)
+    q, k, v = ol.qkv_bias_split(qkv, bias, 12)
+    full = (qkv + bias).view(128, 3, 12, 64)
+    assert torch.equal(q, full[:, 0] * 0.125) and torch.equal(k, full[:, 1]) and torch.equal(v, full[:, 2])
+
+
+def test_layer_composition_matches_plain_torch_modules():
+    """One 12-block sequence forced to full attention == a textbook post-LN encoder layer."""
+    torch.manual_seed(0)
+    g = torch.Generator().manual_seed(0)
+    hid, ffn, heads = 128, 256, 2
+    w = ol.random_layer_weights(hid, ffn, g, std=0.2)
+    n = 4
+    x = torch.randn(n * 64, hid)
+    idx, pos = md.hf_to_index([n * 64], 0, heads)          # n < 12 -> every row lists all blocks
+    got = ol.encoder_layer(x, w, heads, [0, n], idx, pos, heads, eps=1e-5)
+    qkv = x @ w["qkv_weight"] + w["qkv_bias"]
+    q, k, v = (t.view(n * 64, heads, 64).transpose(0, 1) for t in qkv.split(hid, dim=1))
+    ctx = F.scaled_dot_product_attention(q, k, v).transpose(0, 1).reshape(n * 64, hid)
+    a = F.layer_norm(ctx @ w["attn_out_weight"] + w["attn_out_bias"] + x, (hid,), w["attn_ln_weight"], w["attn_ln_bias"], 1e-5)
+    i = F.gelu(a @ w["inter_weight"] + w["inter_bias"], approximate="tanh")
+    want = F.layer_norm(i @ w["out_weight"] + w["out_bias"] + a, (hid,), w["out_ln_weight"], w["out_ln_bias"], 1e-5)
+    assert (got - want).abs().max().item() < 2e-5
