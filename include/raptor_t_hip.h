@@ -1,0 +1,177 @@
+/*
+ * raptor_t_hip.h -- C ABI of the MI355X (gfx950) block-sparse encoder-layer library.
+ *
+ * Drop-in boundary for the hot path of Raptor-T: these are the entry points the
+ * reference's C++ layer functors reach through `layers/kernels/kernel.h` and
+ * `layers/kernels/mat_mul.h`, plus the host metadata the reference builds in
+ * `layers/multi_headed_attention.cpp` and `python/util.py`.  Plain pointers and sizes
+ * only; no torch types, no exceptions, no exit().
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative errno-style code; a text for
+ *     the calling thread's last failure is available from rt_last_error_string();
+ *   - device pointers are borrowed (never freed here) and must belong to the current
+ *     HIP device; `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - `dtype` is an rt_dtype; fp16/bf16 kernels accumulate and normalise in fp32;
+ *   - a packed batch of B sequences is described by `seq_blocks` (B+1 ints): prefix
+ *     sums of the per-sequence counts of 64-token blocks (`seq_len_info` of
+ *     python/util.py:37,45); NB = seq_blocks[B], T = 64 * NB tokens.
+ *
+ * Head-major packed layout (produced by rt_qkv_bias_split, consumed by
+ * rt_bs_attention_fwd): for sequence s (n blocks, first global block g0) and head h
+ * the 64x64 tiles of blocks 0..n-1 start at element (g0*H + h*n) * 4096; Q and K tiles
+ * are row-major [token][d]; a V tile is stored transposed, [d][slot], where slot p of
+ * every group of 16 holds token (p & ~15) | perm(p & 15), perm = {0,1,2,3,8,9,10,11,
+ * 4,5,6,7,12,13,14,15} (the order in which a 32x32 MFMA accumulator hands P back as
+ * the next MFMA's operand).  rt_unpack_v_tiles undoes it for inspection.
+ */
+#ifndef RAPTOR_T_HIP_H
+#define RAPTOR_T_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RT_BLOCK 64           /* tokens per block (bert_attention.h:39) */
+#define RT_HEAD_DIM 64        /* the attention kernel is specialised for d = 64 */
+#define RT_NUM_RAND 3         /* random blocks per row (multi_headed_attention.cpp:27) */
+#define RT_MIN_SPARSE_BLOCKS 12  /* below this a sequence runs full attention
+                                    (python/modeling_big_bird.py:2079-2094) */
+
+typedef enum { RT_F16 = 0, RT_BF16 = 1, RT_F32 = 2 } rt_dtype;
+
+enum {
+  RT_OK = 0,
+  RT_EINVAL = -22,   /* bad argument / shape the kernels do not support */
+  RT_ENOMEM = -12,   /* output capacity too small or allocation failed */
+  RT_EIO = -5,       /* a HIP / hipBLASLt call failed */
+  RT_ENOSYS = -38,   /* combination not implemented */
+  RT_ECANCELED = -125 /* pipeline was terminated */
+};
+
+/* plan modes of rt_meta_build_to_index / rt_pipeline_create */
+enum {
+  RT_PLAN_HF = 0,         /* per-head plan of the reference's oracle, numpy-RNG exact,
+                             seed = layer index (python/modeling_big_bird.py:573-597) */
+  RT_PLAN_REFERENCE = 1,  /* head-shared plan with the row rules of
+                             layers/multi_headed_attention.cpp:44-125, seeded */
+  RT_PLAN_EXPLICIT = 2    /* caller supplies rand_attn */
+};
+/* plan policies (which lengths use the truncated max-length generator) */
+enum { RT_POLICY_REFERENCE_PATCHED = 0, RT_POLICY_HF_UPSTREAM = 1 };
+
+const char* rt_last_error_string(void);
+int rt_abi_version(void);
+
+/* ------------------------------------------------------------------ host metadata */
+
+/* numpy.random.seed(seed) followed by `count` calls of numpy.random.permutation(n_i):
+ * writes the permutations of arange(n_i) back to back.  Exposes the RNG the plans are
+ * drawn with so that it can be checked against numpy itself. */
+int rt_meta_np_permutations(uint32_t seed, const int* n, int count, int* out);
+
+/* Prefix block counts of a batch: replaces the first half of `generate_data_metainfo`
+ * (python/util.py:36-37,45).  seq_lens in tokens, each a positive multiple of 64. */
+int rt_meta_seq_prefix_blocks(const int* seq_lens, int batch, int* out_seq_blocks);
+
+/* rand_attn[heads][n-2][3] for one sequence of `length` tokens, seed = layer index:
+ * replaces python/modeling_big_bird.py:573-597 with :1039-1314. */
+int rt_meta_rand_attn(int length, uint32_t seed, int heads, int max_pos, int policy, int* out);
+
+/* Sizes of the CSR that rt_meta_build_to_index will write. */
+int rt_meta_to_index_size(const int* seq_blocks, int batch, int plan_heads,
+                          int64_t* idx_len, int64_t* pos_len);
+
+/* BigBird to-block CSR of a packed batch: replaces
+ * MultiHeadedAttention::GenerateSparseBlockIndex (layers/multi_headed_attention.cpp:15-140).
+ * Row `hp * NB + g` (plan head hp, global from-block g) lists block ids local to g's
+ * sequence; duplicates are kept.  mode RT_PLAN_HF: plan_heads = heads, rand_attn NULL;
+ * RT_PLAN_REFERENCE: plan_heads = 1; RT_PLAN_EXPLICIT: rand_attn holds, sequence after
+ * sequence (sequences below 12 blocks contribute nothing), [plan_heads][n_s-2][3]. */
+int rt_meta_build_to_index(const int* seq_blocks, int batch, int plan_heads, int mode,
+                           uint32_t seed, int max_pos, int policy, const int* rand_attn,
+                           int* out_idx, int64_t idx_cap, int* out_pos, int64_t pos_cap);
+
+/* Per from-block cost [n,7,8..8,7,n] and total: python/util.py:38-46. */
+int rt_meta_block_costs(const int* seq_blocks, int batch, int* out_costs, int64_t* total);
+
+/* LPT work plan: replaces generate_parition_plan (python/util.py:11-34).
+ * out_pos[n_wg+1], out_ids[heads*NB]; unit id = blk + head*n_s + seq_start*heads. */
+int rt_meta_partition_lpt(const int* seq_blocks, int batch, int heads, int n_wg,
+                          int* out_pos, int* out_ids);
+
+/* --------------------------------------------------------------------- GPU kernels */
+
+/* Replaces kernels::add_bias_and_transpose_kernel (layers/kernels/
+ * add_bias_and_transpose.cu:212-233): qkv[T, 3*H*64] token-major + bias[3*H*64] ->
+ * q (scaled by q_scale), k, vt in the head-major packed layout. */
+int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt,
+                      const int* seq_blocks_dev, int batch, int total_blocks, int heads,
+                      float q_scale, int dtype, void* stream);
+
+/* Inverse of the V-tile layout: vt (packed, transposed) -> v[T, H*64] token-major. */
+int rt_unpack_v_tiles(const void* vt, void* v, const int* seq_blocks_dev, int batch,
+                      int total_blocks, int heads, int dtype, void* stream);
+
+/* Replaces kernels::test_gemm_1 (layers/kernels/sparse_attention.cu:3192-3228) and the
+ * two live kernels behind it (:2953-3190 balanced, :2111-2403 non balanced):
+ * out[T, H*64] token-major = softmax over the listed key blocks of (q . k) @ v, the
+ * scale already folded into q.  to_idx/to_pos: device CSR from rt_meta_build_to_index
+ * (plan_heads = 1 or heads).  If from_idx/from_pos are non-NULL the launch is
+ * `n_wg` persistent workgroups each walking its slice of the LPT plan (balanced);
+ * otherwise one workgroup per (head, from-block) unit. */
+int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out,
+                        const int* seq_blocks_dev, int batch, int total_blocks, int heads,
+                        const int* to_idx, const int* to_pos, int plan_heads,
+                        const int* from_idx, const int* from_pos, int n_wg,
+                        int dtype, void* stream);
+
+/* Replaces kernels::add_bias_and_layernorm_kernel (layers/kernels/
+ * add_bias_and_layernorm.cu:268-285): out = LN(out + bias + residual) * gamma + beta,
+ * in place on out[rows, hidden]; hidden a multiple of 8. */
+int rt_bias_residual_layernorm(void* out, const void* residual, const void* bias,
+                               const void* gamma, const void* beta, int64_t rows, int hidden,
+                               float eps, int dtype, void* stream);
+
+/* Replaces kernels::add_bias_act_kernel (layers/kernels/add_bias_act.cu:114-133):
+ * out = gelu_tanh(out + bias), in place on out[rows, width]; width a multiple of 8. */
+int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype, void* stream);
+
+/* ---------------------------------------------------------------------- dense GEMM */
+
+/* Replaces kernels::MatMul (layers/kernels/mat_mul.cpp:9-96): row-major
+ * C[M,N] = A[M,K] . B[K,N] through hipBLASLt with fp32 accumulation.  The handle owns
+ * the hipBLASLt context, the heuristic cache and a workspace. */
+typedef struct rt_gemm_ctx rt_gemm_ctx;
+int rt_gemm_create(rt_gemm_ctx** ctx);
+int rt_gemm_destroy(rt_gemm_ctx* ctx);
+int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c,
+            int64_t m, int64_t n, int64_t k, int dtype, void* stream);
+
+/* ------------------------------------------------------- metadata / stream pipeline */
+
+/* Replaces Semaphore + MetaData + the per-layer std::async index workers
+ * (layers/semaphore.cpp:8-37, layers/metadata.cpp:6-18,
+ * layers/multi_headed_attention.h:102-103, .cpp:16-139).  One worker thread per layer
+ * waits on a counting semaphore; rt_pipeline_publish stores the batch geometry and
+ * signals every layer; each worker builds its layer's CSR (seed = layer index) into
+ * pinned memory, copies it on a private copy stream and records an event;
+ * rt_pipeline_acquire blocks the host until that layer's CSR is queued, then makes the
+ * caller's stream wait on the event.  device < 0 keeps everything on the host (the
+ * returned pointers are host pointers) so the ordering logic can be exercised without
+ * a GPU.  async = 0 builds the CSR inside rt_pipeline_acquire instead. */
+typedef struct rt_pipeline rt_pipeline;
+int rt_pipeline_create(rt_pipeline** p, int n_layers, int heads, int plan_mode, int max_pos,
+                       int policy, int async, int device);
+int rt_pipeline_publish(rt_pipeline* p, const int* seq_blocks, int batch);
+int rt_pipeline_acquire(rt_pipeline* p, int layer, void* stream, const int** to_idx,
+                        const int** to_pos, int* plan_heads, double* host_wait_us);
+int rt_pipeline_release(rt_pipeline* p, int layer, void* stream);
+int rt_pipeline_destroy(rt_pipeline* p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RAPTOR_T_HIP_H */

@@ -1,0 +1,253 @@
+"""ctypes binding of `libraptor_t_hip.so` (declared in include/raptor_t_hip.h).
+
+Thin by design: numpy arrays for host metadata, `tensor.data_ptr()` for device memory,
+the current torch stream for launches.  Every wrapper raises `RaptorError` with the
+library's own message on a non-zero status.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libraptor_t_hip.so")
+
+RT_F16, RT_BF16, RT_F32 = 0, 1, 2
+RT_PLAN_HF, RT_PLAN_REFERENCE, RT_PLAN_EXPLICIT = 0, 1, 2
+RT_POLICY_REFERENCE_PATCHED, RT_POLICY_HF_UPSTREAM = 0, 1
+RT_EINVAL, RT_ENOMEM, RT_EIO, RT_ENOSYS, RT_ECANCELED = -22, -12, -5, -38, -125
+
+EXPORTS = [
+    "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
+    "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
+    "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_v_tiles", "rt_bs_attention_fwd",
+    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm",
+    "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
+    "rt_pipeline_destroy",
+]
+
+
+class RaptorError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("raptor_t_hip error %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; fails loudly when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("%s is missing: run `make -C raptor-t_amd/csrc` (or __graft_entry__.build())" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        L.rt_last_error_string.restype = ctypes.c_char_p
+        i32p, i64p, vp = ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p
+        I, U, L64, F = ctypes.c_int, ctypes.c_uint32, ctypes.c_int64, ctypes.c_float
+        L.rt_meta_np_permutations.argtypes = [U, i32p, I, i32p]
+        L.rt_meta_seq_prefix_blocks.argtypes = [i32p, I, i32p]
+        L.rt_meta_rand_attn.argtypes = [I, U, I, I, I, i32p]
+        L.rt_meta_to_index_size.argtypes = [i32p, I, I, i64p, i64p]
+        L.rt_meta_build_to_index.argtypes = [i32p, I, I, I, U, I, I, i32p, i32p, L64, i32p, L64]
+        L.rt_meta_block_costs.argtypes = [i32p, I, i32p, i64p]
+        L.rt_meta_partition_lpt.argtypes = [i32p, I, I, I, i32p, i32p]
+        L.rt_qkv_bias_split.argtypes = [vp, vp, vp, vp, vp, vp, I, I, I, F, I, vp]
+        L.rt_unpack_v_tiles.argtypes = [vp, vp, vp, I, I, I, I, vp]
+        L.rt_bs_attention_fwd.argtypes = [vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
+        L.rt_bias_residual_layernorm.argtypes = [vp, vp, vp, vp, vp, L64, I, F, I, vp]
+        L.rt_bias_gelu.argtypes = [vp, vp, L64, I, I, vp]
+        L.rt_gemm_create.argtypes = [ctypes.POINTER(vp)]
+        L.rt_gemm_destroy.argtypes = [vp]
+        L.rt_gemm.argtypes = [vp, vp, vp, vp, L64, L64, L64, I, vp]
+        L.rt_pipeline_create.argtypes = [ctypes.POINTER(vp), I, I, I, I, I, I, I]
+        L.rt_pipeline_publish.argtypes = [vp, i32p, I]
+        L.rt_pipeline_acquire.argtypes = [vp, I, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), i32p,
+                                          ctypes.POINTER(ctypes.c_double)]
+        L.rt_pipeline_release.argtypes = [vp, I, vp]
+        L.rt_pipeline_destroy.argtypes = [vp]
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise RaptorError(rc, lib().rt_last_error_string().decode("utf-8", "replace"))
+
+
+def _i32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int32))
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_int))
+
+
+# ----------------------------------------------------------------------------- host metadata
+def np_permutations(seed, sizes):
+    sizes = _i32(sizes)
+    out = np.empty(int(sizes.sum()), dtype=np.int32)
+    check(lib().rt_meta_np_permutations(seed, _p(sizes), len(sizes), _p(out)))
+    return out
+
+
+def seq_prefix_blocks(seq_lens):
+    lens = _i32(seq_lens)
+    out = np.empty(len(lens) + 1, dtype=np.int32)
+    check(lib().rt_meta_seq_prefix_blocks(_p(lens), len(lens), _p(out)))
+    return out
+
+
+def rand_attn(length, seed, heads, max_pos=4096, policy=RT_POLICY_REFERENCE_PATCHED):
+    n = max(length // 64, 2)
+    out = np.empty((heads, n - 2, 3), dtype=np.int32)
+    check(lib().rt_meta_rand_attn(length, seed, heads, max_pos, policy, _p(out)))
+    return out
+
+
+def to_index_size(seq_blocks, plan_heads):
+    sb = _i32(seq_blocks)
+    a, b = ctypes.c_int64(), ctypes.c_int64()
+    check(lib().rt_meta_to_index_size(_p(sb), len(sb) - 1, plan_heads, ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value
+
+
+def build_to_index(seq_blocks, plan_heads, mode=RT_PLAN_HF, seed=0, max_pos=4096,
+                   policy=RT_POLICY_REFERENCE_PATCHED, rand_attn=None):
+    sb = _i32(seq_blocks)
+    n_idx, n_pos = to_index_size(sb, plan_heads)
+    idx = np.empty(n_idx, dtype=np.int32)
+    pos = np.empty(n_pos, dtype=np.int32)
+    ra = None if rand_attn is None else _i32(rand_attn).reshape(-1)
+    check(lib().rt_meta_build_to_index(_p(sb), len(sb) - 1, plan_heads, mode, seed, max_pos, policy,
+                                       None if ra is None else _p(ra), _p(idx), n_idx, _p(pos), n_pos))
+    return idx, pos
+
+
+def block_costs(seq_blocks):
+    sb = _i32(seq_blocks)
+    out = np.empty(int(sb[-1]), dtype=np.int32)
+    tot = ctypes.c_int64()
+    check(lib().rt_meta_block_costs(_p(sb), len(sb) - 1, _p(out), ctypes.byref(tot)))
+    return out, tot.value
+
+
+def partition_lpt(seq_blocks, heads, n_wg):
+    sb = _i32(seq_blocks)
+    pos = np.empty(n_wg + 1, dtype=np.int32)
+    ids = np.empty(int(sb[-1]) * heads, dtype=np.int32)
+    check(lib().rt_meta_partition_lpt(_p(sb), len(sb) - 1, heads, n_wg, _p(pos), _p(ids)))
+    return pos, ids
+
+
+# ------------------------------------------------------------------------------- GPU kernels
+def _dtype_code(t):
+    import torch
+    return {torch.float16: RT_F16, torch.bfloat16: RT_BF16, torch.float32: RT_F32}[t.dtype]
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dp(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def qkv_bias_split(qkv, bias, q, k, vt, seq_blocks_dev, heads, q_scale):
+    batch = seq_blocks_dev.numel() - 1
+    nb = qkv.shape[0] // 64
+    check(lib().rt_qkv_bias_split(_dp(qkv), _dp(bias), _dp(q), _dp(k), _dp(vt), _dp(seq_blocks_dev), batch, nb,
+                                  heads, q_scale, _dtype_code(qkv), _stream()))
+
+
+def unpack_v_tiles(vt, v, seq_blocks_dev, heads):
+    batch = seq_blocks_dev.numel() - 1
+    nb = v.shape[0] // 64
+    check(lib().rt_unpack_v_tiles(_dp(vt), _dp(v), _dp(seq_blocks_dev), batch, nb, heads, _dtype_code(v), _stream()))
+
+
+def bs_attention_fwd(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads,
+                     from_idx=None, from_pos=None):
+    batch = seq_blocks_dev.numel() - 1
+    nb = out.shape[0] // 64
+    n_wg = 0 if from_pos is None else from_pos.numel() - 1
+    check(lib().rt_bs_attention_fwd(_dp(q), _dp(k), _dp(vt), _dp(out), _dp(seq_blocks_dev), batch, nb, heads,
+                                    _dp(to_idx), _dp(to_pos), plan_heads, _dp(from_idx), _dp(from_pos), n_wg,
+                                    _dtype_code(out), _stream()))
+
+
+def bias_residual_layernorm(out, residual, bias, gamma, beta, eps):
+    rows, hidden = out.shape
+    check(lib().rt_bias_residual_layernorm(_dp(out), _dp(residual), _dp(bias), _dp(gamma), _dp(beta), rows, hidden,
+                                           eps, _dtype_code(out), _stream()))
+
+
+def bias_gelu(out, bias):
+    rows, width = out.shape
+    check(lib().rt_bias_gelu(_dp(out), _dp(bias), rows, width, _dtype_code(out), _stream()))
+
+
+class Gemm:
+    """Owner of one rt_gemm_ctx."""
+
+    def __init__(self):
+        self._h = ctypes.c_void_p()
+        check(lib().rt_gemm_create(ctypes.byref(self._h)))
+
+    def __call__(self, a, b, c):
+        m, k = a.shape
+        n = b.shape[1]
+        check(lib().rt_gemm(self._h, _dp(a), _dp(b), _dp(c), m, n, k, _dtype_code(a), _stream()))
+        return c
+
+    def close(self):
+        if self._h:
+            lib().rt_gemm_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Pipeline:
+    """Owner of one rt_pipeline (device < 0: host only)."""
+
+    def __init__(self, n_layers, heads, plan_mode=RT_PLAN_HF, max_pos=4096, policy=RT_POLICY_REFERENCE_PATCHED,
+                 async_=True, device=0):
+        self._h = ctypes.c_void_p()
+        self.device = device
+        check(lib().rt_pipeline_create(ctypes.byref(self._h), n_layers, heads, plan_mode, max_pos, policy,
+                                       1 if async_ else 0, device))
+
+    def publish(self, seq_blocks):
+        sb = _i32(seq_blocks)
+        check(lib().rt_pipeline_publish(self._h, _p(sb), len(sb) - 1))
+
+    def acquire(self, layer, stream=None):
+        idx, pos = ctypes.c_void_p(), ctypes.c_void_p()
+        ph, wait = ctypes.c_int(), ctypes.c_double()
+        st = ctypes.c_void_p(0) if self.device < 0 else (stream if stream is not None else _stream())
+        check(lib().rt_pipeline_acquire(self._h, layer, st, ctypes.byref(idx), ctypes.byref(pos), ctypes.byref(ph),
+                                        ctypes.byref(wait)))
+        return idx.value, pos.value, ph.value, wait.value
+
+    def release(self, layer, stream=None):
+        st = ctypes.c_void_p(0) if self.device < 0 else (stream if stream is not None else _stream())
+        check(lib().rt_pipeline_release(self._h, layer, st))
+
+    def close(self):
+        if self._h:
+            lib().rt_pipeline_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

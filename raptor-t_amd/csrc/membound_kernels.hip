@@ -1,0 +1,402 @@
+// Memory-bound kernels of the encoder layer for gfx950 (wave64): fused
+// bias+residual+LayerNorm, bias+GELU(tanh form), and the QKV bias/scale/head split that
+// writes the head-major packed layout the attention kernel reads.
+//
+// All three move 16 bytes per lane per access so that every wave issues full 1 KiB
+// requests; statistics and the activation are computed in fp32.
+//
+// Replaces, from the reference: layers/kernels/add_bias_and_layernorm.cu:191-285,
+// layers/kernels/add_bias_act.cu:41-48,86-133, layers/kernels/add_bias_and_transpose.cu:118-233.
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "rt_common.h"
+
+namespace {
+
+// ---- 16-byte vectors of the storage type <-> 8 (or 4) floats --------------------------
+template <typename T> struct Vec;            // VEC = elements per 16 bytes
+template <> struct Vec<__half> {
+  static constexpr int N = 8;
+  __device__ static void load(const __half* p, float* f) {
+    uint4 r = *reinterpret_cast<const uint4*>(p);
+    const __half2* h = reinterpret_cast<const __half2*>(&r);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { float2 t = __half22float2(h[i]); f[2 * i] = t.x; f[2 * i + 1] = t.y; }
+  }
+  __device__ static void store(__half* p, const float* f) {
+    uint4 r;
+    __half2* h = reinterpret_cast<__half2*>(&r);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h[i] = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+    *reinterpret_cast<uint4*>(p) = r;
+  }
+};
+template <> struct Vec<__hip_bfloat16> {
+  static constexpr int N = 8;
+  __device__ static void load(const __hip_bfloat16* p, float* f) {
+    uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(&r);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { f[2 * i] = __uint_as_float(w[i] << 16); f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+  }
+  __device__ static uint32_t rne(float x) {          // float -> bf16 bits, round to nearest even
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;   // keep NaN a NaN
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  }
+  __device__ static void store(__hip_bfloat16* p, const float* f) {
+    uint4 r;
+    uint32_t* w = reinterpret_cast<uint32_t*>(&r);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = rne(f[2 * i]) | (rne(f[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4*>(p) = r;
+  }
+};
+template <> struct Vec<float> {
+  static constexpr int N = 4;
+  __device__ static void load(const float* p, float* f) {
+    float4 r = *reinterpret_cast<const float4*>(p);
+    f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
+  }
+  __device__ static void store(float* p, const float* f) {
+    *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+  }
+};
+
+template <int G> __device__ inline float group_sum(float v) {   // sum over G consecutive lanes
+#pragma unroll
+  for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// ---- bias + residual + LayerNorm ------------------------------------------------------
+// One row per group of G lanes (G = 32 or 64); each lane keeps CHUNKS 16-byte chunks of
+// the row in registers: hidden = CHUNKS * G * Vec<T>::N.  Two passes over registers.
+template <typename T, int CHUNKS, int G>
+__global__ __launch_bounds__(256) void bias_residual_layernorm_kernel(
+    T* __restrict__ out, const T* __restrict__ residual, const T* __restrict__ bias,
+    const T* __restrict__ gamma, const T* __restrict__ beta, int64_t rows, float eps) {
+  constexpr int N = Vec<T>::N;
+  constexpr int HIDDEN = CHUNKS * G * N;
+  const int lane = threadIdx.x % G;
+  const int64_t row = int64_t(blockIdx.x) * (256 / G) + threadIdx.x / G;
+  if (row >= rows) return;
+  T* o = out + row * HIDDEN;
+  const T* r = residual + row * HIDDEN;
+  float x[CHUNKS][N];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int col = (c * G + lane) * N;
+    float a[N], b[N], d[N];
+    Vec<T>::load(o + col, a);
+    Vec<T>::load(r + col, b);
+    Vec<T>::load(bias + col, d);
+#pragma unroll
+    for (int i = 0; i < N; ++i) { x[c][i] = a[i] + d[i] + b[i]; sum += x[c][i]; }
+  }
+  const float mean = group_sum<G>(sum) * (1.0f / HIDDEN);
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+    for (int i = 0; i < N; ++i) { const float t = x[c][i] - mean; sq += t * t; }
+  const float rstd = rsqrtf(group_sum<G>(sq) * (1.0f / HIDDEN) + eps);
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int col = (c * G + lane) * N;
+    float g[N], b[N], y[N];
+    Vec<T>::load(gamma + col, g);
+    Vec<T>::load(beta + col, b);
+#pragma unroll
+    for (int i = 0; i < N; ++i) y[i] = (x[c][i] - mean) * rstd * g[i] + b[i];
+    Vec<T>::store(o + col, y);
+  }
+}
+
+// Any hidden that is a multiple of the vector width: one wave per row, three sweeps.
+template <typename T>
+__global__ __launch_bounds__(256) void bias_residual_layernorm_generic_kernel(
+    T* __restrict__ out, const T* __restrict__ residual, const T* __restrict__ bias,
+    const T* __restrict__ gamma, const T* __restrict__ beta, int64_t rows, int hidden, float eps) {
+  constexpr int N = Vec<T>::N;
+  const int lane = threadIdx.x % 64;
+  const int64_t row = int64_t(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (row >= rows) return;
+  T* o = out + row * hidden;
+  const T* r = residual + row * hidden;
+  float sum = 0.f;
+  for (int col = lane * N; col < hidden; col += 64 * N) {
+    float a[N], b[N], d[N];
+    Vec<T>::load(o + col, a); Vec<T>::load(r + col, b); Vec<T>::load(bias + col, d);
+#pragma unroll
+    for (int i = 0; i < N; ++i) sum += a[i] + d[i] + b[i];
+  }
+  const float mean = group_sum<64>(sum) / hidden;
+  float sq = 0.f;
+  for (int col = lane * N; col < hidden; col += 64 * N) {
+    float a[N], b[N], d[N];
+    Vec<T>::load(o + col, a); Vec<T>::load(r + col, b); Vec<T>::load(bias + col, d);
+#pragma unroll
+    for (int i = 0; i < N; ++i) { const float t = a[i] + d[i] + b[i] - mean; sq += t * t; }
+  }
+  const float rstd = rsqrtf(group_sum<64>(sq) / hidden + eps);
+  for (int col = lane * N; col < hidden; col += 64 * N) {
+    float a[N], b[N], d[N], g[N], be[N], y[N];
+    Vec<T>::load(o + col, a); Vec<T>::load(r + col, b); Vec<T>::load(bias + col, d);
+    Vec<T>::load(gamma + col, g); Vec<T>::load(beta + col, be);
+#pragma unroll
+    for (int i = 0; i < N; ++i) y[i] = (a[i] + d[i] + b[i] - mean) * rstd * g[i] + be[i];
+    Vec<T>::store(o + col, y);
+  }
+}
+
+template <typename T, int CHUNKS, int G>
+void launch_ln(T* out, const T* res, const T* bias, const T* gamma, const T* beta, int64_t rows, float eps,
+               hipStream_t st) {
+  const int rows_per_wg = 256 / G;
+  const unsigned grid = unsigned((rows + rows_per_wg - 1) / rows_per_wg);
+  hipLaunchKernelGGL((bias_residual_layernorm_kernel<T, CHUNKS, G>), dim3(grid), dim3(256), 0, st, out, res, bias,
+                     gamma, beta, rows, eps);
+}
+
+template <typename T>
+int ln_dispatch(void* out, const void* res, const void* bias, const void* gamma, const void* beta, int64_t rows,
+                int hidden, float eps, hipStream_t st) {
+  T* o = static_cast<T*>(out);
+  const T *r = static_cast<const T*>(res), *b = static_cast<const T*>(bias), *g = static_cast<const T*>(gamma),
+          *be = static_cast<const T*>(beta);
+  constexpr int N = Vec<T>::N;
+  const int per32 = 32 * N;
+  if (hidden % per32 == 0) {
+    switch (hidden / per32) {        // chunks per lane with 32 lanes per row
+      case 1: launch_ln<T, 1, 32>(o, r, b, g, be, rows, eps, st); return RT_OK;
+      case 2: launch_ln<T, 2, 32>(o, r, b, g, be, rows, eps, st); return RT_OK;
+      case 3: launch_ln<T, 3, 32>(o, r, b, g, be, rows, eps, st); return RT_OK;   // 768 (fp16/bf16)
+      case 4: launch_ln<T, 4, 32>(o, r, b, g, be, rows, eps, st); return RT_OK;   // 1024
+      case 6: launch_ln<T, 3, 64>(o, r, b, g, be, rows, eps, st); return RT_OK;
+      case 8: launch_ln<T, 4, 64>(o, r, b, g, be, rows, eps, st); return RT_OK;
+      case 12: launch_ln<T, 6, 64>(o, r, b, g, be, rows, eps, st); return RT_OK;
+      case 16: launch_ln<T, 8, 64>(o, r, b, g, be, rows, eps, st); return RT_OK;
+      default: break;
+    }
+  }
+  const unsigned grid = unsigned((rows + 3) / 4);
+  hipLaunchKernelGGL((bias_residual_layernorm_generic_kernel<T>), dim3(grid), dim3(256), 0, st, o, r, b, g, be, rows,
+                     hidden, eps);
+  return RT_OK;
+}
+
+// ---- bias + GELU (tanh form) ------------------------------------------------------------
+// gelu(x) = 0.5 x (1 + tanh(u)), u = c0 (x + c1 x^3)  ==  x / (1 + exp(-2u)).
+__device__ inline float gelu_tanh(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return x * __frcp_rn(1.0f + __expf(-2.0f * u));
+}
+
+// The launch makes the grid stride a multiple of the row width, so a thread always lands
+// in the same column: its bias chunk is loaded once and no index division is needed in
+// the loop.  Four independent 16-byte loads are issued before any of them is used.
+template <typename T>
+__global__ __launch_bounds__(256) void bias_gelu_kernel(T* __restrict__ out, const T* __restrict__ bias,
+                                                        int64_t n_vec, int width_vec) {
+  constexpr int N = Vec<T>::N;
+  constexpr int U = 4;
+  const int64_t stride = int64_t(gridDim.x) * 256;
+  int64_t v = int64_t(blockIdx.x) * 256 + threadIdx.x;
+  float b[N];
+  Vec<T>::load(bias + int(v % width_vec) * N, b);
+  for (; v + (U - 1) * stride < n_vec; v += U * stride) {
+    float a[U][N];
+#pragma unroll
+    for (int u = 0; u < U; ++u) Vec<T>::load(out + (v + u * stride) * N, a[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) a[u][i] = gelu_tanh(a[u][i] + b[i]);
+      Vec<T>::store(out + (v + u * stride) * N, a[u]);
+    }
+  }
+  for (; v < n_vec; v += stride) {
+    float a[N];
+    Vec<T>::load(out + v * N, a);
+#pragma unroll
+    for (int i = 0; i < N; ++i) a[i] = gelu_tanh(a[i] + b[i]);
+    Vec<T>::store(out + v * N, a);
+  }
+}
+
+// ---- QKV bias + scale + head split --------------------------------------------------------
+// Workgroup (g, h): global block g, head h.  Q and K tiles are copied row-major; the V
+// tile goes through LDS and is written transposed with the MFMA slot order.
+__device__ inline int find_seq(const int* __restrict__ seq_blocks, int batch, int g) {
+  int lo = 0, hi = batch;                   // seq_blocks[lo] <= g < seq_blocks[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (seq_blocks[mid] <= g) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__device__ inline int slot_token(int p) {   // token held by slot p of a transposed V tile
+  const int e = p & 15;
+  return (p & ~15) | ((e & 3) | ((e & 4) << 1) | ((e & 8) >> 1));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
+                                                             T* __restrict__ q, T* __restrict__ k,
+                                                             T* __restrict__ vt, const int* __restrict__ seq_blocks,
+                                                             int batch, int heads, float q_scale) {
+  constexpr int N = Vec<T>::N;              // elements per 16 bytes
+  constexpr int CPR = 64 / N;               // 16-byte chunks per 64-wide row
+  __shared__ float vtile[64][65];
+  const int g = blockIdx.x, h = blockIdx.y;
+  const int s = find_seq(seq_blocks, batch, g);
+  const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
+  const int64_t tile = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
+  const int dm = heads * 64;
+  const T* src = qkv + int64_t(g) * 64 * (3 * dm) + h * 64;
+  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
+    const int row = c / CPR, col = (c % CPR) * N;
+    float x[N], b[N];
+    Vec<T>::load(src + int64_t(row) * 3 * dm + col, x);
+    Vec<T>::load(bias + h * 64 + col, b);
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] = (x[i] + b[i]) * q_scale;
+    Vec<T>::store(q + tile + row * 64 + col, x);
+    Vec<T>::load(src + int64_t(row) * 3 * dm + dm + col, x);
+    Vec<T>::load(bias + dm + h * 64 + col, b);
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] += b[i];
+    Vec<T>::store(k + tile + row * 64 + col, x);
+    Vec<T>::load(src + int64_t(row) * 3 * dm + 2 * dm + col, x);
+    Vec<T>::load(bias + 2 * dm + h * 64 + col, b);
+#pragma unroll
+    for (int i = 0; i < N; ++i) vtile[row][col + i] = x[i] + b[i];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
+    const int d = c / CPR, p0 = (c % CPR) * N;
+    float x[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) x[i] = vtile[slot_token(p0 + i)][d];
+    Vec<T>::store(vt + tile + d * 64 + p0, x);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void unpack_v_tiles_kernel(const T* __restrict__ vt, T* __restrict__ v,
+                                                             const int* __restrict__ seq_blocks, int batch,
+                                                             int heads) {
+  const int g = blockIdx.x, h = blockIdx.y;
+  const int s = find_seq(seq_blocks, batch, g);
+  const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
+  const int64_t tile = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
+  const int dm = heads * 64;
+  for (int e = threadIdx.x; e < 4096; e += 256) {
+    const int d = e / 64, p = e % 64;
+    v[(int64_t(g) * 64 + slot_token(p)) * dm + h * 64 + d] = vt[tile + e];
+  }
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return rt::fail(RT_EIO, "%s launch failed: %s", what, hipGetErrorString(e));
+  return RT_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int rt_bias_residual_layernorm(void* out, const void* residual, const void* bias, const void* gamma,
+                               const void* beta, int64_t rows, int hidden, float eps, int dtype, void* stream) {
+  RT_REQUIRE(out && residual && bias && gamma && beta, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(rows >= 0 && rows < (int64_t(1) << 31), RT_EINVAL, "rows=%lld out of range", (long long)rows);
+  const int n = dtype == RT_F32 ? 4 : 8;
+  RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
+  RT_REQUIRE(hidden > 0 && hidden % n == 0, RT_EINVAL, "hidden=%d must be a positive multiple of %d", hidden, n);
+  RT_REQUIRE(aligned16(out) && aligned16(residual) && aligned16(bias) && aligned16(gamma) && aligned16(beta),
+             RT_EINVAL, "pointers must be 16-byte aligned");
+  if (rows == 0) return RT_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == RT_F16) ln_dispatch<__half>(out, residual, bias, gamma, beta, rows, hidden, eps, st);
+  else if (dtype == RT_BF16) ln_dispatch<__hip_bfloat16>(out, residual, bias, gamma, beta, rows, hidden, eps, st);
+  else ln_dispatch<float>(out, residual, bias, gamma, beta, rows, hidden, eps, st);
+  return check_launch("bias_residual_layernorm");
+}
+
+int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype, void* stream) {
+  RT_REQUIRE(out && bias, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
+  const int n = dtype == RT_F32 ? 4 : 8;
+  RT_REQUIRE(rows >= 0 && width > 0 && width % n == 0, RT_EINVAL, "rows=%lld width=%d: width must be a positive multiple of %d",
+             (long long)rows, width, n);
+  RT_REQUIRE(aligned16(out) && aligned16(bias), RT_EINVAL, "pointers must be 16-byte aligned");
+  if (rows == 0) return RT_OK;
+  const int64_t n_vec = rows * (width / n);
+  const int width_vec = width / n;
+  int a = 256, b = width_vec;                       // m = width_vec / gcd(256, width_vec)
+  while (b) { const int t = a % b; a = b; b = t; }
+  const int64_t m = width_vec / a;
+  int64_t want = (n_vec + 256 * 4 - 1) / (256 * 4);           // about four vectors per thread
+  if (want > 256 * 16) want = 256 * 16;                       // 16 workgroups per CU, grid-stride beyond
+  want = (want + m - 1) / m * m;                              // stride % width_vec == 0
+  const unsigned grid = unsigned(want);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == RT_F16)
+    hipLaunchKernelGGL(bias_gelu_kernel<__half>, dim3(grid), dim3(256), 0, st, (__half*)out, (const __half*)bias, n_vec, width / n);
+  else if (dtype == RT_BF16)
+    hipLaunchKernelGGL(bias_gelu_kernel<__hip_bfloat16>, dim3(grid), dim3(256), 0, st, (__hip_bfloat16*)out, (const __hip_bfloat16*)bias, n_vec, width / n);
+  else
+    hipLaunchKernelGGL(bias_gelu_kernel<float>, dim3(grid), dim3(256), 0, st, (float*)out, (const float*)bias, n_vec, width / n);
+  return check_launch("bias_gelu");
+}
+
+int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt, const int* seq_blocks_dev,
+                      int batch, int total_blocks, int heads, float q_scale, int dtype, void* stream) {
+  RT_REQUIRE(qkv && bias && q && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && heads <= 65535, RT_EINVAL,
+             "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
+  RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
+  RT_REQUIRE(aligned16(qkv) && aligned16(bias) && aligned16(q) && aligned16(k) && aligned16(vt), RT_EINVAL,
+             "pointers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  dim3 grid(total_blocks, heads);
+  if (dtype == RT_F16)
+    hipLaunchKernelGGL(qkv_bias_split_kernel<__half>, grid, dim3(256), 0, st, (const __half*)qkv, (const __half*)bias,
+                       (__half*)q, (__half*)k, (__half*)vt, seq_blocks_dev, batch, heads, q_scale);
+  else if (dtype == RT_BF16)
+    hipLaunchKernelGGL(qkv_bias_split_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)qkv,
+                       (const __hip_bfloat16*)bias, (__hip_bfloat16*)q, (__hip_bfloat16*)k, (__hip_bfloat16*)vt,
+                       seq_blocks_dev, batch, heads, q_scale);
+  else
+    hipLaunchKernelGGL(qkv_bias_split_kernel<float>, grid, dim3(256), 0, st, (const float*)qkv, (const float*)bias,
+                       (float*)q, (float*)k, (float*)vt, seq_blocks_dev, batch, heads, q_scale);
+  return check_launch("qkv_bias_split");
+}
+
+int rt_unpack_v_tiles(const void* vt, void* v, const int* seq_blocks_dev, int batch, int total_blocks, int heads,
+                      int dtype, void* stream) {
+  RT_REQUIRE(vt && v && seq_blocks_dev, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && heads <= 65535, RT_EINVAL,
+             "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  dim3 grid(total_blocks, heads);
+  if (dtype == RT_F16)
+    hipLaunchKernelGGL(unpack_v_tiles_kernel<__half>, grid, dim3(256), 0, st, (const __half*)vt, (__half*)v, seq_blocks_dev, batch, heads);
+  else if (dtype == RT_BF16)
+    hipLaunchKernelGGL(unpack_v_tiles_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)vt, (__hip_bfloat16*)v, seq_blocks_dev, batch, heads);
+  else if (dtype == RT_F32)
+    hipLaunchKernelGGL(unpack_v_tiles_kernel<float>, grid, dim3(256), 0, st, (const float*)vt, (float*)v, seq_blocks_dev, batch, heads);
+  else
+    return rt::fail(RT_EINVAL, "unknown dtype %d", dtype);
+  return check_launch("unpack_v_tiles");
+}
+
+}  // extern "C"

@@ -1,0 +1,92 @@
+"""Shared helpers of the GPU parity tests and of `__graft_entry__.smoke()`: drive the
+C-ABI through `raptor_t_amd.capi` and compare with the CPU oracle.  Not collected by
+pytest (no test_ prefix)."""
+import math
+
+import numpy as np
+import torch
+
+from oracle import attention as oa
+from oracle import layer as ol
+from oracle import metadata as md
+
+SLOT_PERM = [0, 1, 2, 3, 8, 9, 10, 11, 4, 5, 6, 7, 12, 13, 14, 15]
+
+
+def slot_tokens():
+    return torch.tensor([(p & ~15) | SLOT_PERM[p & 15] for p in range(64)], dtype=torch.long)
+
+
+def pack_heads(x, seq_blocks, transpose_v=False):
+    """Token-major [T, H, d] -> the head-major packed layout as a flat tensor (torch statement
+    of the layout documented in include/raptor_t_hip.h)."""
+    t, heads, d = x.shape
+    parts = []
+    st = slot_tokens().to(x.device)
+    for s in range(len(seq_blocks) - 1):
+        n = int(seq_blocks[s + 1] - seq_blocks[s])
+        blk = x[int(seq_blocks[s]) * 64: int(seq_blocks[s + 1]) * 64].view(n, 64, heads, d).permute(2, 0, 1, 3)
+        if transpose_v:
+            blk = blk[:, :, st, :].transpose(2, 3)          # [H, n, d, slot]
+        parts.append(blk.contiguous().view(-1))
+    return torch.cat(parts)
+
+
+def device_plan(capi, seq_lens, heads, seed=0, mode=None, plan_heads=None, device="cuda"):
+    sb = capi.seq_prefix_blocks(seq_lens)
+    mode = capi.RT_PLAN_HF if mode is None else mode
+    ph = (1 if mode == capi.RT_PLAN_REFERENCE else heads) if plan_heads is None else plan_heads
+    idx, pos = capi.build_to_index(sb, ph, mode=mode, seed=seed)
+    dev = lambda a: torch.from_numpy(a).to(device)
+    return sb, idx, pos, ph, dev(sb), dev(idx), dev(pos)
+
+
+def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0):
+    """q, k, v: [T, H, 64] CUDA tensors (q unscaled).  Returns (gpu_out [T, H*64], oracle fp32)."""
+    sb, idx, pos, ph, sb_d, idx_d, pos_d = device_plan(capi, seq_lens, heads, seed, mode)
+    qs = (q.float() * 0.125).to(q.dtype)
+    qp, kp = pack_heads(qs, sb), pack_heads(k, sb)
+    vp = pack_heads(v, sb, transpose_v=True)
+    out = torch.full((q.shape[0], heads * 64), float("nan"), dtype=q.dtype, device=q.device)
+    from_idx = from_pos = None
+    if n_wg:
+        fp, fi = capi.partition_lpt(sb, heads, n_wg)
+        from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
+    capi.bs_attention_fwd(qp, kp, vp, out, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos)
+    torch.cuda.synchronize()
+    ref = oa.csr_attention(qs.cpu(), k.cpu(), v.cpu(), sb.tolist(), idx, pos, ph, scale=1.0)
+    return out, ref
+
+
+def run_layer_case(pkg, seq_lens, hidden, heads, ffn, dtype, seed=0, eps=1e-5, n_wg=0):
+    """One encoder layer through the C-ABI on cuda:0 against the oracle; returns max abs error."""
+    capi = pkg.capi
+    g = torch.Generator().manual_seed(seed)
+    w32 = ol.random_layer_weights(hidden, ffn, g)
+    t = sum(seq_lens)
+    x32 = torch.randn(t, hidden, generator=g)
+    w = {k_: v_.to(dtype).cuda() for k_, v_ in w32.items()}
+    x = x32.to(dtype).cuda()
+    sb, idx, pos, ph, sb_d, idx_d, pos_d = device_plan(capi, seq_lens, heads, seed)
+    gemm = capi.Gemm()
+    new = lambda *shape: torch.empty(*shape, dtype=dtype, device="cuda")
+    qkv, q, k, vt = new(t, 3 * hidden), new(t * hidden), new(t * hidden), new(t * hidden)
+    ctx, attn, inter, out = new(t, hidden), new(t, hidden), new(t, ffn), new(t, hidden)
+    from_idx = from_pos = None
+    if n_wg:
+        fp, fi = capi.partition_lpt(sb, heads, n_wg)
+        from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
+    gemm(x, w["qkv_weight"], qkv)
+    capi.qkv_bias_split(qkv, w["qkv_bias"], q, k, vt, sb_d, heads, 1.0 / math.sqrt(hidden // heads))
+    capi.bs_attention_fwd(q, k, vt, ctx, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos)
+    gemm(ctx, w["attn_out_weight"], attn)
+    capi.bias_residual_layernorm(attn, x, w["attn_out_bias"], w["attn_ln_weight"], w["attn_ln_bias"], eps)
+    gemm(attn, w["inter_weight"], inter)
+    capi.bias_gelu(inter, w["inter_bias"])
+    gemm(inter, w["out_weight"], out)
+    capi.bias_residual_layernorm(out, attn, w["out_bias"], w["out_ln_weight"], w["out_ln_bias"], eps)
+    torch.cuda.synchronize()
+    gemm.close()
+    wr = {k_: v_.to(dtype).float() for k_, v_ in w32.items()}          # the oracle sees the rounded weights
+    want = ol.encoder_layer(x32.to(dtype).float(), wr, heads, sb.tolist(), idx, pos, ph, eps)
+    return (out.float().cpu() - want).abs().max().item()
