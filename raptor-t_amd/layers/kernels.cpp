@@ -1,0 +1,168 @@
+#include "kernels.h"
+
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <mutex>
+#include <stdexcept>
+
+namespace sparse_transformers {
+namespace layers {
+namespace kernels {
+
+void* current_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+int dtype_code(const torch::Tensor& t) {
+  switch (t.scalar_type()) {
+    case torch::kHalf: return RT_F16;
+    case torch::kBFloat16: return RT_BF16;
+    case torch::kFloat: return RT_F32;
+    default: throw std::invalid_argument("unsupported tensor dtype (fp16, bf16 or fp32 expected)");
+  }
+}
+
+void check(int rc, const char* what) {
+  if (rc != RT_OK) throw std::runtime_error(std::string(what) + ": " + rt_last_error_string());
+}
+
+rt_gemm_ctx* shared_gemm_handle() {
+  static std::mutex m;
+  static rt_gemm_ctx* ctx = nullptr;
+  std::lock_guard<std::mutex> lk(m);
+  if (!ctx) check(rt_gemm_create(&ctx), "rt_gemm_create");
+  return ctx;
+}
+
+static void require_cuda_contiguous(const torch::Tensor& t, const char* name) {
+  if (!t.is_cuda() || !t.is_contiguous())
+    throw std::invalid_argument(std::string(name) + " must be a contiguous GPU tensor");
+}
+
+ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* key) {
+  auto it = info.find(key);
+  if (it == info.end()) return;
+  slot_ = &it->second;
+  hipEvent_t a, b;
+  if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { slot_ = nullptr; return; }
+  start_ = a;
+  stop_ = b;
+  (void)hipEventRecord(a, static_cast<hipStream_t>(current_stream()));
+}
+
+ScopedGpuTimer::~ScopedGpuTimer() {
+  if (!slot_) return;
+  hipEvent_t a = static_cast<hipEvent_t>(start_), b = static_cast<hipEvent_t>(stop_);
+  (void)hipEventRecord(b, static_cast<hipStream_t>(current_stream()));
+  (void)hipEventSynchronize(b);
+  float ms = 0.f;
+  if (hipEventElapsedTime(&ms, a, b) == hipSuccess) *slot_ += ms * 1000.0f;
+  (void)hipEventDestroy(a);
+  (void)hipEventDestroy(b);
+}
+
+void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b_trans, float alpha,
+            torch::Tensor& out, float beta, rt_gemm_ctx* handle, const std::string& name) {
+  if (a_trans || b_trans || alpha != 1.0f || beta != 0.0f)
+    throw std::invalid_argument(name + ": only out = A . B is supported");
+  require_cuda_contiguous(A, "A");
+  require_cuda_contiguous(B, "B");
+  require_cuda_contiguous(out, "out");
+  if (A.dim() != 2 || B.dim() != 2 || A.size(1) != B.size(0) || out.numel() != A.size(0) * B.size(1))
+    throw std::invalid_argument(name + ": shape mismatch");
+  check(rt_gemm(handle, A.data_ptr(), B.data_ptr(), out.data_ptr(), A.size(0), B.size(1), A.size(1), dtype_code(A),
+                current_stream()), name.c_str());
+}
+
+void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,
+                                   torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,
+                                   int batch_size, int head_num, int block_num, int head_size,
+                                   std::map<std::string, float>& info, bool kernel_fusion) {
+  ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel");
+  if (head_size != RT_HEAD_DIM) throw std::invalid_argument("head size must be 64");
+  const float scale = 1.0f / std::sqrt(float(head_size));
+  if (kernel_fusion) {
+    check(rt_qkv_bias_split(input_data.data_ptr(), bias.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                            seq_len_info_tensor.data_ptr<int>(), batch_size, block_num, head_num, scale,
+                            dtype_code(input_data), current_stream()), "rt_qkv_bias_split");
+    return;
+  }
+  // Unfused: library ops, one sequence at a time (the reference's own fallback is a
+  // reshape/permute chain, add_bias_and_transpose.cu:219-222).
+  auto sb = seq_len_info_tensor.cpu();
+  const int* s = sb.data_ptr<int>();
+  const int64_t dm = int64_t(head_num) * head_size;
+  auto x = input_data + bias;
+  static const int perm16[16] = {0, 1, 2, 3, 8, 9, 10, 11, 4, 5, 6, 7, 12, 13, 14, 15};
+  std::vector<int64_t> slots(64);
+  for (int p = 0; p < 64; ++p) slots[p] = (p & ~15) | perm16[p & 15];
+  auto slot_idx = torch::tensor(slots, torch::kLong).to(x.device());
+  auto qf = q.view({-1}), kf = k.view({-1}), vf = v.view({-1});
+  for (int b = 0; b < batch_size; ++b) {
+    const int64_t n = s[b + 1] - s[b], t0 = int64_t(s[b]) * 64, off = t0 * dm;
+    auto seq = x.narrow(0, t0, n * 64);
+    auto qs = (seq.narrow(1, 0, dm) * scale).view({n, 64, head_num, head_size}).permute({2, 0, 1, 3});
+    auto ks = seq.narrow(1, dm, dm).view({n, 64, head_num, head_size}).permute({2, 0, 1, 3});
+    auto vs = seq.narrow(1, 2 * dm, dm).view({n, 64, head_num, head_size}).permute({2, 0, 1, 3});
+    qf.narrow(0, off, n * 64 * dm).copy_(qs.contiguous().view({-1}));
+    kf.narrow(0, off, n * 64 * dm).copy_(ks.contiguous().view({-1}));
+    vf.narrow(0, off, n * 64 * dm).copy_(vs.index_select(2, slot_idx).transpose(2, 3).contiguous().view({-1}));
+  }
+}
+
+void add_bias_and_layernorm_kernel(torch::Tensor& out, const torch::Tensor& input_data, const torch::Tensor& bias,
+                                   int seq_len, int normalized_len, float eps, const torch::Tensor& layernorm_weight,
+                                   const torch::Tensor& layernorm_bias, std::map<std::string, float>& info,
+                                   bool kernel_fusion) {
+  ScopedGpuTimer timer(info, "add_bias_and_layernorm_kernel");
+  if (kernel_fusion) {
+    check(rt_bias_residual_layernorm(out.data_ptr(), input_data.data_ptr(), bias.data_ptr(),
+                                     layernorm_weight.data_ptr(), layernorm_bias.data_ptr(), seq_len, normalized_len,
+                                     eps, dtype_code(out), current_stream()), "rt_bias_residual_layernorm");
+    return;
+  }
+  // Unfused: three library launches (add_bias_and_layernorm.cu:276-279)
+  out.add_(input_data).add_(bias);
+  out.copy_(torch::layer_norm(out, {normalized_len}, layernorm_weight, layernorm_bias, eps));
+}
+
+void add_bias_act_kernel(const torch::Tensor& bias, torch::Tensor& out, int total_seq_len, int dim_size,
+                         std::map<std::string, float>& info, bool kernel_fusion) {
+  ScopedGpuTimer timer(info, "add_bias_act_kernel");
+  if (kernel_fusion) {
+    check(rt_bias_gelu(out.data_ptr(), bias.data_ptr(), total_seq_len, dim_size, dtype_code(out), current_stream()),
+          "rt_bias_gelu");
+    return;
+  }
+  // Unfused: add then the tanh-form GELU (the reference's fallback uses the erf form here,
+  // an inconsistency with its fused kernel; add_bias_act.cu:123-126)
+  out.add_(bias);
+  out.copy_(torch::gelu(out, "tanh"));
+}
+
+void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torch::Tensor& v, torch::Tensor& out,
+                      int batch_size, const torch::Tensor& seq_len_info_tensor, const torch::Tensor& from_select_index,
+                      const torch::Tensor& from_select_index_position, const int* to_select_index,
+                      const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
+                      int head_num, std::map<std::string, float>& info, bool balanced) {
+  ScopedGpuTimer timer(info, "attention");
+  const int* from_idx = nullptr;
+  const int* from_pos = nullptr;
+  int n_wg = 0;
+  if (balanced) {
+    if (from_select_index_position.numel() != int64_t(block_limit) + 1)
+      throw std::invalid_argument("balanced attention: the plan has a different number of workgroups than block_limit");
+    if (from_select_index.numel() != int64_t(block_num) * head_num)
+      throw std::invalid_argument("balanced attention: the plan does not cover every (head, block) unit");
+    from_idx = from_select_index.data_ptr<int>();
+    from_pos = from_select_index_position.data_ptr<int>();
+    n_wg = block_limit;
+  }
+  check(rt_bs_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), seq_len_info_tensor.data_ptr<int>(),
+                            batch_size, block_num, head_num, to_select_index, to_select_index_position, plan_heads,
+                            from_idx, from_pos, n_wg, dtype_code(out), current_stream()), "rt_bs_attention_fwd");
+}
+
+}  // namespace kernels
+}  // namespace layers
+}  // namespace sparse_transformers

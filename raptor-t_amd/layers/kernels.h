@@ -1,0 +1,72 @@
+// Tensor-level launchers used by the layer functors: the names and argument meaning of
+// layers/kernels/kernel.h and layers/kernels/mat_mul.h of the reference, each a thin
+// shim over the C ABI in include/raptor_t_hip.h (which is where the GPU code lives).
+//
+// `info`: a key that the caller has pre-seeded is accumulated with the GPU time of the
+// call in microseconds, measured with HIP events on the current stream (the reference
+// takes host wall-clock around an asynchronous launch, which only means something under
+// CUDA_LAUNCH_BLOCKING=1; layers/kernels/add_bias_act.cu:129-132).
+#pragma once
+#include <torch/torch.h>
+
+#include <map>
+#include <string>
+
+#include "../../include/raptor_t_hip.h"
+
+namespace sparse_transformers {
+namespace layers {
+namespace kernels {
+
+enum class ActivationType { Gelu = 0, Tanh = 1, Relu = 2 };
+
+void* current_stream();
+int dtype_code(const torch::Tensor& t);
+void check(int rc, const char* what);
+// One hipBLASLt context (heuristic cache + workspace) shared by every layer of the process;
+// the reference creates a cuBLAS handle per layer object (multi_headed_attention.h:94).
+rt_gemm_ctx* shared_gemm_handle();
+
+// RAII timer: accumulates into info[key] only when the key already exists.
+class ScopedGpuTimer {
+ public:
+  ScopedGpuTimer(std::map<std::string, float>& info, const char* key);
+  ~ScopedGpuTimer();
+
+ private:
+  float* slot_ = nullptr;
+  void* start_ = nullptr;
+  void* stop_ = nullptr;
+};
+
+// kernels::MatMul (layers/kernels/mat_mul.cpp:9-96): out[M,N] = A[M,K] . B[K,N]; only the
+// no-transpose, alpha = 1, beta = 0 form the layers use is supported.
+void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b_trans, float alpha,
+            torch::Tensor& out, float beta, rt_gemm_ctx* handle, const std::string& name);
+
+// layers/kernels/add_bias_and_transpose.cu:212-233
+void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,
+                                   torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,
+                                   int batch_size, int head_num, int block_num, int head_size,
+                                   std::map<std::string, float>& info, bool kernel_fusion);
+
+// layers/kernels/add_bias_and_layernorm.cu:268-285
+void add_bias_and_layernorm_kernel(torch::Tensor& out, const torch::Tensor& input_data, const torch::Tensor& bias,
+                                   int seq_len, int normalized_len, float eps, const torch::Tensor& layernorm_weight,
+                                   const torch::Tensor& layernorm_bias, std::map<std::string, float>& info,
+                                   bool kernel_fusion);
+
+// layers/kernels/add_bias_act.cu:114-133
+void add_bias_act_kernel(const torch::Tensor& bias, torch::Tensor& out, int total_seq_len, int dim_size,
+                         std::map<std::string, float>& info, bool kernel_fusion);
+
+// kernels::test_gemm_1 (layers/kernels/sparse_attention.cu:3192-3228): block-sparse attention
+void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torch::Tensor& v, torch::Tensor& out,
+                      int batch_size, const torch::Tensor& seq_len_info_tensor, const torch::Tensor& from_select_index,
+                      const torch::Tensor& from_select_index_position, const int* to_select_index,
+                      const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
+                      int head_num, std::map<std::string, float>& info, bool balanced);
+
+}  // namespace kernels
+}  // namespace layers
+}  // namespace sparse_transformers

@@ -1,0 +1,255 @@
+"""Python callers of the `raptor_t` layer functors.
+
+Mirrors python/modeling_bert.py of the reference: the same classes (`BertEmbeddings`,
+`BertIntermediate`, `BertOutput`, `BertAttention`, `BertLayer`, `BertEncoder`,
+`BertModelNoPooler`), the same call order and buffer aliasing (attention writes
+`attention_output`; the FFN writes back into the layer's input buffer, :204-207), the same
+weight re-layout in `from_torch` (`cat(q, k, v).t()`, `dense.weight.t()`, :137-163).
+Differences: sizes are read from the weights (no 768 / 3072 literals), LayerNorm eps and
+the dtype are arguments, and `from_weights` builds layers from plain tensors so that a
+random-init model needs no HuggingFace object.
+"""
+import os
+import sys
+from typing import Optional, Sequence
+
+import torch
+import torch.nn as nn
+
+_LIB = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+if _LIB not in sys.path:
+    sys.path.insert(0, _LIB)
+try:
+    import raptor_t as cxx          # built by raptor-t_amd/layers/build_ext.py
+except ImportError as e:            # no silent fallback: the layer API is the product
+    raise ImportError("the raptor_t extension is not built: run __graft_entry__.build() (%s)" % e)
+
+roctx = torch.cuda.nvtx             # torch maps these ranges onto roctx on ROCm
+
+
+def to_param_dict(torch_module: torch.nn.Module):
+    return {k: v for k, v in torch_module.named_parameters()}
+
+
+def create_empty_if_none(tensor, shape, device, dtype=torch.float16):
+    if tensor is None:
+        tensor = torch.zeros(shape, dtype=dtype, device=device)
+    return tensor
+
+
+class BertEmbeddings:
+    """Word + position + token-type embeddings and LayerNorm(eps 1e-12), kept in PyTorch as in
+    the reference (:27-69); returns the packed [T, D] activations in the encoder's dtype."""
+
+    def __init__(self, word_embeddings_weight, position_embeddings_weight, token_type_embeddings_weight,
+                 layerNorm_weight, layerNorm_bias, pad_token_id: int = 0, dtype=torch.float16, device="cuda"):
+        self.word_embeddings = nn.Embedding.from_pretrained(word_embeddings_weight.detach().float(), freeze=True,
+                                                            padding_idx=pad_token_id).to(device)
+        self.position_embeddings = nn.Embedding.from_pretrained(position_embeddings_weight.detach().float(),
+                                                                freeze=True).to(device)
+        self.token_type_embeddings = nn.Embedding.from_pretrained(token_type_embeddings_weight.detach().float(),
+                                                                  freeze=True).to(device)
+        hidden = word_embeddings_weight.shape[1]
+        self.LayerNorm = nn.LayerNorm(hidden, eps=1e-12).to(device)
+        with torch.no_grad():
+            self.LayerNorm.weight.copy_(layerNorm_weight)
+            self.LayerNorm.bias.copy_(layerNorm_bias)
+        self.dtype = dtype
+
+    @torch.no_grad()
+    def __call__(self, input_ids=None, position_ids=None, token_type_ids=None, output=None):
+        if input_ids is None or position_ids is None or token_type_ids is None:
+            raise ValueError("input_ids, position_ids and token_type_ids are all required")
+        emb = (self.word_embeddings(input_ids.long()) + self.token_type_embeddings(token_type_ids.long())
+               + self.position_embeddings(position_ids.long()))
+        return self.LayerNorm(emb).to(self.dtype).contiguous()
+
+    @staticmethod
+    def from_torch(bert_embedding, dtype=torch.float16):
+        p = to_param_dict(bert_embedding)
+        return BertEmbeddings(p["word_embeddings.weight"], p["position_embeddings.weight"],
+                              p["token_type_embeddings.weight"], p["LayerNorm.weight"], p["LayerNorm.bias"],
+                              dtype=dtype)
+
+
+class BertIntermediate(cxx.BertIntermediate):
+    def __call__(self, input_tensor, total_seq_len, output=None, kernel_fusion=True, test_info=None):
+        roctx.range_push("intermediate")
+        test_info = {} if test_info is None else test_info
+        test_info = super().__call__(input_tensor, output, test_info, kernel_fusion)
+        roctx.range_pop()
+        return test_info
+
+    @staticmethod
+    def from_weights(weight_in_out, bias):
+        return BertIntermediate(weight_in_out.contiguous(), bias.contiguous())
+
+    @staticmethod
+    def from_torch(intermediate, dtype=torch.float16):
+        p = to_param_dict(intermediate)
+        return BertIntermediate(torch.t(p["dense.weight"]).contiguous().to(dtype).cuda(), p["dense.bias"].to(dtype).cuda())
+
+
+class BertOutput(cxx.BertOutput):
+    def __call__(self, intermediate_output, attention_output, total_seq_len, output=None, kernel_fusion=True,
+                 test_info=None):
+        roctx.range_push("output")
+        test_info = {} if test_info is None else test_info
+        test_info = super().__call__(intermediate_output, attention_output, output, test_info, kernel_fusion)
+        roctx.range_pop()
+        return test_info
+
+    @staticmethod
+    def from_torch(output, dtype=torch.float16, eps=1e-5):
+        p = to_param_dict(output)
+        c = lambda t: t.detach().to(dtype).cuda().contiguous()
+        return BertOutput(c(torch.t(p["dense.weight"])), c(p["dense.bias"]), c(p["LayerNorm.weight"]),
+                          c(p["LayerNorm.bias"]), eps)
+
+
+class BertAttention(cxx.BertAttention):
+    def __call__(self, input_tensor, seq_position_info, seq_position_info_tensor, partition_part_index_tensor,
+                 partition_part_tensor, context_layer, block_limit, attention_mask=None, head_mask=None,
+                 output_attentions=False, is_trans_weight=False, kernel_fusion=True, test_info=None, balanced=True):
+        roctx.range_push("attention")
+        test_info = {} if test_info is None else test_info
+        if attention_mask is None:
+            attention_mask = torch.empty(0)
+        test_info = super().__call__(input_tensor, attention_mask, context_layer, seq_position_info,
+                                     seq_position_info_tensor, partition_part_index_tensor, partition_part_tensor,
+                                     block_limit, test_info, kernel_fusion, balanced)
+        roctx.range_pop()
+        return test_info
+
+    @staticmethod
+    def from_torch(attention, layer_idx: int, async_: bool, dtype=torch.float16, eps=1e-5):
+        p = {k: v for k, v in attention.named_parameters()}
+        c = lambda t: t.detach().to(dtype).cuda().contiguous()
+        with torch.no_grad():
+            qkv_weight = torch.t(torch.cat((p["self.query.weight"], p["self.key.weight"], p["self.value.weight"]), 0))
+            qkv_bias = torch.cat((p["self.query.bias"], p["self.key.bias"], p["self.value.bias"]), 0)
+            return BertAttention(c(qkv_weight), c(qkv_bias), c(torch.t(p["output.dense.weight"])),
+                                 c(p["output.dense.bias"]), c(p["output.LayerNorm.weight"]),
+                                 c(p["output.LayerNorm.bias"]), attention.self.num_attention_heads, layer_idx, async_, eps)
+
+
+class BertLayer:
+    def __init__(self, attention: BertAttention, intermediate: BertIntermediate, output: BertOutput):
+        self.attention = attention
+        self.intermediate = intermediate
+        self.output = output
+
+    def __call__(self, hidden_states, seq_position_info, seq_position_info_tensor, partition_part_index_tensor,
+                 partition_part_tensor, intermediate_temp, output_layer_temp, attention_output, block_limit,
+                 attention_mask=None, head_mask=None, output_attentions=False, kernel_fusion=True, test_info=None,
+                 balanced=True):
+        roctx.range_push("layer")
+        total = seq_position_info[-1] * 64
+        test_info = self.attention(hidden_states, seq_position_info, seq_position_info_tensor,
+                                   partition_part_index_tensor, partition_part_tensor, attention_output, block_limit,
+                                   attention_mask, head_mask, output_attentions=output_attentions, test_info=test_info,
+                                   kernel_fusion=kernel_fusion, balanced=balanced)
+        test_info = self.intermediate(attention_output, total, intermediate_temp, test_info=test_info,
+                                      kernel_fusion=kernel_fusion)
+        test_info = self.output(intermediate_temp, attention_output, total, hidden_states, test_info=test_info,
+                                kernel_fusion=kernel_fusion)
+        roctx.range_pop()
+        return hidden_states, test_info
+
+    @staticmethod
+    def from_weights(w, heads, layer_idx, async_=True, eps=1e-5):
+        """`w`: the twelve tensors of one layer in the `[in, out]` layout (keys as
+        produced by `random_layer_weights`)."""
+        att = BertAttention(w["qkv_weight"], w["qkv_bias"], w["attn_out_weight"], w["attn_out_bias"],
+                            w["attn_ln_weight"], w["attn_ln_bias"], heads, layer_idx, async_, eps)
+        inter = BertIntermediate(w["inter_weight"], w["inter_bias"])
+        out = BertOutput(w["out_weight"], w["out_bias"], w["out_ln_weight"], w["out_ln_bias"], eps)
+        return BertLayer(att, inter, out)
+
+    @staticmethod
+    def from_torch(layer, layer_idx: int, async_: bool, dtype=torch.float16, eps=1e-5):
+        return BertLayer(BertAttention.from_torch(layer.attention, layer_idx, async_, dtype, eps),
+                         BertIntermediate.from_torch(layer.intermediate, dtype),
+                         BertOutput.from_torch(layer.output, dtype, eps))
+
+
+class BertEncoder:
+    def __init__(self, layer: Sequence[BertLayer]):
+        self.layer = layer
+
+    def __call__(self, hidden_states, total_seq_len, thread_block_limit, seq_position_info, seq_position_info_tensor,
+                 partition_part_index_tensor, partition_part_tensor, output_layer_temp, intermediate_temp,
+                 attention_output, test_info=None, kernel_fusion=True, balanced=True, attention_mask=None,
+                 head_mask=None, output_attentions=False, output_hidden_states=False):
+        for l in self.layer:
+            hidden_states, test_info = l(hidden_states=hidden_states, block_limit=thread_block_limit,
+                                         seq_position_info=seq_position_info,
+                                         seq_position_info_tensor=seq_position_info_tensor,
+                                         partition_part_index_tensor=partition_part_index_tensor,
+                                         partition_part_tensor=partition_part_tensor,
+                                         output_layer_temp=output_layer_temp, intermediate_temp=intermediate_temp,
+                                         attention_output=attention_output, attention_mask=attention_mask,
+                                         test_info=test_info, kernel_fusion=kernel_fusion,
+                                         output_attentions=output_attentions, balanced=balanced)
+        return hidden_states, test_info
+
+    @staticmethod
+    def from_weights(layers_w, heads, async_=True, eps=1e-5):
+        return BertEncoder([BertLayer.from_weights(w, heads, i, async_, eps) for i, w in enumerate(layers_w)])
+
+    @staticmethod
+    def from_torch(encoder, async_: bool, dtype=torch.float16, eps=1e-5):
+        return BertEncoder([BertLayer.from_torch(l, i, async_, dtype, eps) for i, l in enumerate(encoder.layer)])
+
+
+class BertModelNoPooler:
+    def __init__(self, embeddings: BertEmbeddings, encoder: BertEncoder):
+        self.embeddings = embeddings
+        self.encoder = encoder
+
+    def __call__(self, inputs, total_seq_len, thread_block_limit, seq_position_info, seq_position_info_tensor,
+                 partition_part_index_tensor, partition_part_tensor, attention_masks=None, token_type_ids=None,
+                 position_ids=None, output_layer_temp=None, intermediate_temp=None, attention_output=None,
+                 test_info=None, kernel_fusion=True, balanced=True, **unused):
+        roctx.range_push("embeddings")
+        hidden = self.embeddings(inputs, position_ids=position_ids, token_type_ids=token_type_ids)
+        roctx.range_pop()
+        d = hidden.shape[1]
+        dev, dt = hidden.device, hidden.dtype
+        output_layer_temp = create_empty_if_none(output_layer_temp, (total_seq_len, d), dev, dt)
+        attention_output = create_empty_if_none(attention_output, (total_seq_len, d), dev, dt)
+        if intermediate_temp is None:
+            raise ValueError("intermediate_temp [T, F] must be provided (its width defines the FFN size)")
+        roctx.range_push("encoder")
+        out, test_info = self.encoder(hidden_states=hidden, total_seq_len=total_seq_len,
+                                      thread_block_limit=thread_block_limit, seq_position_info=seq_position_info,
+                                      seq_position_info_tensor=seq_position_info_tensor,
+                                      partition_part_index_tensor=partition_part_index_tensor,
+                                      partition_part_tensor=partition_part_tensor, output_layer_temp=output_layer_temp,
+                                      intermediate_temp=intermediate_temp, attention_output=attention_output,
+                                      test_info={} if test_info is None else test_info, kernel_fusion=kernel_fusion,
+                                      balanced=balanced)
+        roctx.range_pop()
+        return out, test_info
+
+    @staticmethod
+    def from_torch(model, async_: bool = True, dtype=torch.float16, eps=None):
+        eps = model.config.layer_norm_eps if eps is None else eps
+        return BertModelNoPooler(BertEmbeddings.from_torch(model.embeddings, dtype),
+                                 BertEncoder.from_torch(model.encoder, async_, dtype, eps))
+
+
+def random_layer_weights(hidden, ffn, generator, std=0.02, dtype=torch.float16, device="cuda"):
+    """N(0, std) weights and biases in the `[in, out]` layout, gamma = 1, beta = 0."""
+    def n(*shape):
+        return (torch.randn(*shape, generator=generator) * std).to(dtype).to(device)
+    one = lambda k: torch.ones(k, dtype=dtype, device=device)
+    zero = lambda k: torch.zeros(k, dtype=dtype, device=device)
+    return {
+        "qkv_weight": n(hidden, 3 * hidden), "qkv_bias": n(3 * hidden),
+        "attn_out_weight": n(hidden, hidden), "attn_out_bias": n(hidden),
+        "attn_ln_weight": one(hidden), "attn_ln_bias": zero(hidden),
+        "inter_weight": n(hidden, ffn), "inter_bias": n(ffn),
+        "out_weight": n(ffn, hidden), "out_bias": n(hidden),
+        "out_ln_weight": one(hidden), "out_ln_bias": zero(hidden),
+    }

@@ -1,0 +1,155 @@
+"""GPU parity tests of the drop-in layer API (the `raptor_t` pybind module and its Python
+callers) against the CPU oracle and against the HuggingFace BigBird model installed on the
+box, on the same seeded inputs and the same random-block plan."""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+import __graft_entry__ as graft
+from oracle import layer as ol
+from oracle import metadata as md
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    p = graft.load_package()
+    p.capi.lib()
+    assert torch.cuda.is_available()
+    return p
+
+
+@pytest.fixture(scope="module")
+def mb(pkg):
+    return importlib.import_module("raptor_t_amd.modeling_bert")
+
+
+@pytest.fixture(scope="module")
+def ut(pkg):
+    return importlib.import_module("raptor_t_amd.util")
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype):
+    sb = md.seq_prefix_blocks(seq_lens)
+    h = x32.to(dtype).float()
+    for li, w in enumerate(layers_w32):
+        wr = {k: v.to(dtype).float() for k, v in w.items()}
+        idx, pos = md.hf_to_index(seq_lens, li, heads)
+        h = ol.encoder_layer(h, wr, heads, sb, idx, pos, heads, eps)
+    return h
+
+
+@pytest.mark.parametrize("async_,balanced,dtype,hidden,heads,ffn", [
+    (True, True, torch.float16, 768, 12, 3072),
+    (False, False, torch.float16, 768, 12, 3072),
+    (True, True, torch.bfloat16, 1024, 16, 4096),
+])
+def test_encoder_through_layer_api_matches_oracle(mb, ut, async_, balanced, dtype, hidden, heads, ffn):
+    say("encoder api", async_, balanced, dtype, hidden)
+    n_layers, eps, block_limit = 2, 1e-5, 96
+    g = torch.Generator().manual_seed(0)
+    layers_w32 = [ol.random_layer_weights(hidden, ffn, g) for _ in range(n_layers)]
+    layers_w = [{k: v.to(dtype).cuda() for k, v in w.items()} for w in layers_w32]
+    enc = mb.BertEncoder.from_weights(layers_w, heads, async_=async_, eps=eps)
+    meta = mb.cxx.MetaData()
+    worst = 0.0
+    for seq_lens in ([832, 1024, 256], [1280, 768]):       # two batches through the same objects
+        t = sum(seq_lens)
+        x32 = torch.randn(t, hidden, generator=g)
+        hidden_states = x32.to(dtype).cuda()
+        spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, block_limit, heads)
+        meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+        new = lambda w: torch.empty(t, w, dtype=dtype, device="cuda")
+        inter, tmp, attn = new(ffn), new(hidden), new(hidden)
+        info = {"pre_process": 0.0, "attention": 0.0}
+        out, info = enc(hidden_states, t, block_limit, spi, spi_t, ppi_t, pp_t, tmp, inter, attn, test_info=info,
+                        balanced=balanced)
+        torch.cuda.synchronize()
+        assert out.data_ptr() == hidden_states.data_ptr()       # FFN writes back into the layer input buffer
+        assert info["attention"] > 0.0 and info["pre_process"] >= 0.0
+        want = _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype)
+        err = (out.float().cpu() - want).abs().max().item()
+        say("  err", err, "info", info)
+        worst = max(worst, err)
+    meta.terminate_thread()
+    assert worst <= (2e-2 if dtype == torch.float16 else 8e-2)   # bf16: one ulp at |y| ~ 4 is 3e-2
+
+
+def test_fused_and_unfused_paths_agree(mb, ut):
+    say("fusion switch")
+    hidden, heads, ffn, dtype = 768, 12, 3072, torch.float16
+    g = torch.Generator().manual_seed(1)
+    w = {k: v.to(dtype).cuda() for k, v in ol.random_layer_weights(hidden, ffn, g).items()}
+    layer = mb.BertLayer.from_weights(w, heads, 0, async_=True)
+    meta = mb.cxx.MetaData()
+    seq_lens = [896, 320]
+    t = sum(seq_lens)
+    x = torch.randn(t, hidden, generator=g).to(dtype).cuda()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, 64, heads)
+    outs = []
+    for fused in (True, False):
+        meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+        h = x.clone()
+        new = lambda wd: torch.empty(t, wd, dtype=dtype, device="cuda")
+        out, _ = layer(h, spi, spi_t, ppi_t, pp_t, new(ffn), new(hidden), new(hidden), 64, kernel_fusion=fused)
+        torch.cuda.synchronize()
+        outs.append(out.float().cpu())
+    meta.terminate_thread()
+    assert (outs[0] - outs[1]).abs().max().item() <= 2e-2
+
+
+def test_api_rejects_mismatched_batch(mb, ut):
+    hidden, heads, ffn, dtype = 768, 12, 3072, torch.float16
+    g = torch.Generator().manual_seed(2)
+    w = {k: v.to(dtype).cuda() for k, v in ol.random_layer_weights(hidden, ffn, g).items()}
+    layer = mb.BertLayer.from_weights(w, heads, 0, async_=True)
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo([768], 64, 32, heads)
+    meta.update_meta_data(768, spi[-1] + 1, total_comp, spi)
+    x = torch.zeros(832, hidden, dtype=dtype, device="cuda")
+    new = lambda wd: torch.empty(832, wd, dtype=dtype, device="cuda")
+    with pytest.raises((ValueError, RuntimeError)):
+        layer(x, spi, spi_t, ppi_t, pp_t, new(ffn), new(hidden), new(hidden), 32)
+    with pytest.raises((ValueError, RuntimeError)):
+        meta.update_meta_data(100, 0, 0, [0, 12])
+    with pytest.raises((ValueError, RuntimeError)):
+        mb.cxx.BertAttention(torch.zeros(768, 100), torch.zeros(2304), torch.zeros(768, 768), torch.zeros(768),
+                             torch.ones(768), torch.zeros(768), 12, 0, True)
+    meta.terminate_thread()
+
+
+@pytest.mark.parametrize("length", [1024, 832])
+def test_from_torch_matches_huggingface_bigbird(mb, ut, length):
+    """The HuggingFace BigBird model itself (random init, fp32, train mode so that its random
+    blocks are drawn, all dropout at 0) against BertModelNoPooler.from_torch in fp16."""
+    say("hf parity", length)
+    from transformers import BigBirdConfig, BigBirdModel
+    torch.manual_seed(0)
+    cfg = BigBirdConfig(vocab_size=1000, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        intermediate_size=256, max_position_embeddings=4096, attention_type="block_sparse",
+                        block_size=64, num_random_blocks=3, hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+    hf = BigBirdModel(cfg, add_pooling_layer=False).cuda().train()
+    ids = torch.randint(1, 1000, (1, length), device="cuda")
+    with torch.no_grad():
+        want = hf(input_ids=ids).last_hidden_state[0].float().cpu()
+    model = mb.BertModelNoPooler.from_torch(hf, async_=True, dtype=torch.float16)
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo([length], 64, 48, 2)
+    meta.update_meta_data(length, spi[-1] + 1, total_comp, spi)
+    pos = torch.arange(length, device="cuda")
+    inter = torch.empty(length, 256, dtype=torch.float16, device="cuda")
+    out, _ = model(ids[0], length, 48, spi, spi_t, ppi_t, pp_t, token_type_ids=torch.zeros_like(pos),
+                   position_ids=pos, intermediate_temp=inter)
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    err = (out.float().cpu() - want).abs().max().item()
+    say("  hf err", err)
+    assert err <= 2e-2
