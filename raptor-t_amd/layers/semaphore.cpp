@@ -29,6 +29,7 @@ void Semaphore::register_layer(int layer_idx, int heads, bool async) {
   std::lock_guard<std::mutex> lk(mutex_);
   layer_cond[layer_idx] = heads;
   async_ = async;
+  terminate_single = false;      // a newly built layer re-arms a terminated pipeline
 }
 
 void Semaphore::set_plan(int plan_mode, int policy, int max_pos) {
@@ -87,6 +88,8 @@ void Semaphore::Release(int layer_idx, void* stream) {
 void Semaphore::terminate() {
   std::lock_guard<std::mutex> lk(mutex_);
   terminate_single = true;
+  last_batch_.clear();
+  layer_cond.clear();
   if (pipeline_) { rt_pipeline_destroy(pipeline_); pipeline_ = nullptr; }
 }
 
