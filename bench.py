@@ -1,0 +1,253 @@
+"""Benchmark of the block-sparse encoder hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|ref_e2e]
+
+Default workload `c3` is BASELINE.json's config 3: the 12-layer BigBird-base fp16 encoder
+on a padding-free batch of 16 sequences with lengths uniform in [512, 4096] (multiples of
+64, numpy default_rng(0)), random-init N(0, 0.02) weights, N(0, 1) inputs, driven through
+the drop-in layer API (`raptor_t` pybind module) with the asynchronous metadata pipeline.
+One step = MetaData.update_meta_data + one 12-layer forward; inputs are resident in HBM.
+Prints ONE JSON line: seqs/s (value), ms/step, ms/layer, the roofline of the dominant
+hand-written kernel (block-sparse attention, MFMA bound) measured live with HIP events
+inside the timed steps, HBM rooflines of the LayerNorm / GELU / split kernels, and the
+CPU baseline (the oracle layer timed on the host cores on a bounded sample).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+import __graft_entry__ as graft  # noqa: E402
+
+MFMA_PEAK = {"f16": 2.5e15, "bf16": 2.5e15}       # MI355X dense matrix peak, FLOP/s
+HBM_PEAK = 8.0e12                                   # B/s
+PAIR_FLOP = 4 * 64 * 64 * 64                        # QK^T + PV of one (from-block, to-block) pair, d = 64
+METRIC = "seqs/sec + ms/layer, BigBird-base fp16 var-len<=4096; attn MFMA %, LN HBM GB/s"
+
+
+def block_pairs(seq_blocks, heads):
+    tot = 0
+    for s in range(len(seq_blocks) - 1):
+        n = seq_blocks[s + 1] - seq_blocks[s]
+        tot += n * n if n < 12 else 10 * n - 18
+    return tot * heads
+
+
+def hbm_roofline(name, bytes_per_launch, us_per_launch):
+    ach = bytes_per_launch / (us_per_launch * 1e-6)
+    return {"kernel": name, "bound": "hbm", "achieved": ach / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": ach / HBM_PEAK, "traffic": None}
+
+
+def cpu_baseline_layer(seq_lens, hidden, heads, ffn, layers, sample_seqs, reps=3):
+    """Oracle encoder layer (PyTorch-CPU fp32, the reference oracle's algorithm) on the first
+    `sample_seqs` sequences of the batch, scaled by tokens to the whole batch and by the layer
+    count to the whole encoder."""
+    from oracle import layer as ol
+    from oracle import metadata as md
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    lens = list(seq_lens[:sample_seqs])
+    g = torch.Generator().manual_seed(0)
+    w = ol.random_layer_weights(hidden, ffn, g)
+    x = torch.randn(sum(lens), hidden, generator=g)
+    sb = md.seq_prefix_blocks(lens)
+    idx, pos = md.hf_to_index(lens, 0, heads)
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        ol.encoder_layer(x, w, heads, sb, idx, pos, heads)
+        times.append(time.perf_counter() - t0)
+    t_layer = float(np.median(times))
+    t_batch = t_layer * (sum(seq_lens) / sum(lens)) * layers
+    return {"value": len(seq_lens) / t_batch, "unit": "seqs/s", "cores": cores, "kind": "port",
+            "sample": "oracle encoder layer (torch CPU fp32) on the first %d sequences (%d tokens), median of %d, "
+                      "scaled by tokens to the batch and x%d layers; %.2f s per sampled layer"
+                      % (len(lens), sum(lens), reps, layers, t_layer)}
+
+
+def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos=4096):
+    pkg = graft.load_package()
+    mb = importlib.import_module("raptor_t_amd.modeling_bert")
+    ut = importlib.import_module("raptor_t_amd.util")
+    dt = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    g = torch.Generator().manual_seed(0)
+    layers_w = [mb.random_layer_weights(hidden, ffn, g, dtype=dt) for _ in range(layers)]
+    mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, max_pos)
+    enc = mb.BertEncoder.from_weights(layers_w, heads, async_=not args.sync_index, eps=1e-5)
+    meta = mb.cxx.MetaData()
+    t = sum(seq_lens)
+    block_limit = args.block_limit
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, block_limit, heads)
+    x0 = torch.randn(t, hidden, generator=g).to(dt).cuda()
+    hidden_states = torch.empty_like(x0)
+    new = lambda w: torch.empty(t, w, dtype=dt, device="cuda")
+    inter, tmp, attn = new(ffn), new(hidden), new(hidden)
+
+    def step():
+        hidden_states.copy_(x0)
+        meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+        enc(hidden_states, t, block_limit, spi, spi_t, ppi_t, pp_t, tmp, inter, attn, test_info={},
+            balanced=not args.unbalanced)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    mb.cxx.timing_begin()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timing = mb.cxx.timing_collect()
+    meta.terminate_thread()
+
+    ms_step = elapsed / args.steps * 1e3
+    per = {k: v[0] / v[1] for k, v in timing.items() if v[1]}
+    pairs = block_pairs(spi, heads)
+    att_us = per["attention"]
+    att_flops = pairs * PAIR_FLOP
+    ach = att_flops / (att_us * 1e-6)
+    sz = 2
+    out = {
+        "metric": METRIC, "value": len(seq_lens) / (elapsed / args.steps), "unit": "seqs/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step, "ms_per_layer": ms_step / layers,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": name, "layers": layers, "hidden": hidden, "heads": heads, "ffn": ffn,
+                   "batch": len(seq_lens), "tokens": t, "seq_lens": seq_lens, "block_limit": block_limit,
+                   "balanced": not args.unbalanced, "async_index": not args.sync_index,
+                   "weights": "random N(0,0.02)", "plan": "per-head HF plan, seed = layer index"},
+        "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12,
+                     "peak": MFMA_PEAK[dtype] / 1e12, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK[dtype],
+                     "traffic": None, "flop_per_launch": att_flops, "block_pairs": pairs, "us_per_launch": att_us},
+        "roofline_layernorm": hbm_roofline("bias_residual_layernorm_kernel", 3 * t * hidden * sz,
+                                           per["add_bias_and_layernorm_kernel"]),
+        "roofline_gelu": hbm_roofline("bias_gelu_kernel", 2 * t * ffn * sz, per["add_bias_act_kernel"]),
+        "roofline_qkv_split": hbm_roofline("qkv_bias_split_kernel", 2 * t * 3 * hidden * sz,
+                                           per["add_bias_and_transpose_kernel"]),
+        "kernel_us_per_launch": per,
+        "kernel_us_per_step": {k: v[0] / args.steps for k, v in timing.items()},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_layer(seq_lens, hidden, heads, ffn, layers, args.cpu_sample_seqs)
+    return out
+
+
+def time_kernel(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return float(np.median([a.elapsed_time(b) for a, b in evs])) * 1e3      # microseconds
+
+
+def run_attention_only(args):
+    """BASELINE config 2: isolated block-sparse attention, batch 8 x 4096 tokens, 12 heads, fp16."""
+    capi = graft.load_package().capi
+    heads, lens = 12, [4096] * 8
+    t = sum(lens)
+    sb = capi.seq_prefix_blocks(lens)
+    idx, pos = capi.build_to_index(sb, heads, seed=0)
+    dev = lambda a: torch.from_numpy(a).cuda()
+    sb_d, idx_d, pos_d = dev(sb), dev(idx), dev(pos)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    qkv = torch.randn(t, 3 * heads * 64, generator=g, device="cuda", dtype=torch.float16)
+    bias = torch.zeros(3 * heads * 64, device="cuda", dtype=torch.float16)
+    q, k, vt = (torch.empty(t * heads * 64, device="cuda", dtype=torch.float16) for _ in range(3))
+    capi.qkv_bias_split(qkv, bias, q, k, vt, sb_d, heads, capi.Q_SCALE)
+    out = torch.empty(t, heads * 64, device="cuda", dtype=torch.float16)
+    fp, fi = capi.partition_lpt(sb, heads, args.block_limit)
+    fp_d, fi_d = dev(fp), dev(fi)
+    if args.unbalanced:
+        fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads)
+    else:
+        fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads, fi_d, fp_d)
+    us = time_kernel(fn, args.steps, args.warmup)
+    pairs = block_pairs(sb.tolist(), heads)
+    ach = pairs * PAIR_FLOP / (us * 1e-6)
+    return {"metric": "isolated block-sparse attention, batch 8 x 4096, 12 heads x 64, fp16", "value": ach / 1e12,
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": us / 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "c2 isolated attention", "block_pairs": pairs, "block_limit": args.block_limit,
+                       "balanced": not args.unbalanced},
+            "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12, "peak": 2500.0,
+                         "unit": "TFLOP/s", "frac": ach / 2.5e15, "traffic": None}}
+
+
+def run_membound_sweep(args):
+    """BASELINE config 4: LayerNorm and GELU epilogues over tokens {8K, 32K, 64K}, fp16 and bf16."""
+    capi = graft.load_package().capi
+    rows = []
+    for dt, name in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+        for t in (8192, 32768, 65536):
+            g = torch.Generator(device="cuda").manual_seed(0)
+            rn = lambda *s: torch.randn(*s, generator=g, device="cuda").to(dt)
+            x, r, b, ga, be = rn(t, 768), rn(t, 768), rn(768), rn(768), rn(768)
+            us = time_kernel(lambda: capi.bias_residual_layernorm(x, r, b, ga, be, 1e-5), args.steps, args.warmup)
+            rows.append(dict(hbm_roofline("bias_residual_layernorm_kernel", 3 * t * 768 * 2, us), tokens=t, dtype=name, us=us))
+            y, b2 = rn(t, 3072), rn(3072)
+            us = time_kernel(lambda: capi.bias_gelu(y, b2), args.steps, args.warmup)
+            rows.append(dict(hbm_roofline("bias_gelu_kernel", 2 * t * 3072 * 2, us), tokens=t, dtype=name, us=us))
+    best_ln = max(r["frac"] for r in rows if r["kernel"].startswith("bias_residual"))
+    return {"metric": "fused add-bias+LayerNorm / bias+GELU achieved HBM GB/s", "value": best_ln * 8000.0, "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16/bf16", "data": "synthetic",
+            "config": {"workload": "c4 memory-bound op sweep"}, "sweep": rows}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=["c3", "c2", "c4", "c5", "ref_e2e"])
+    ap.add_argument("--block-limit", type=int, default=1024, help="persistent workgroups of the balanced attention launch")
+    ap.add_argument("--unbalanced", action="store_true", help="one workgroup per (head, from-block) unit")
+    ap.add_argument("--sync-index", action="store_true", help="build the block index inline instead of on the workers")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-seqs", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (every sequence is independent; see DESIGN.md for how the batch "
+              "would shard); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    ut = importlib.import_module("raptor_t_amd.util") if graft.load_package() else None
+    if args.workload == "c3":
+        res = run_encoder(args, "c3: 12-layer BigBird-base, batch 16, len U[512,4096]", 768, 12, 3072, 12, "f16",
+                          ut.uniform_lengths(16, 512, 4096, seed=0))
+    elif args.workload == "c5":
+        res = run_encoder(args, "c5: 24-layer BigBird-large shape, batch 4, len U[2048,16384], bf16", 1024, 16, 4096,
+                          24, "bf16", ut.uniform_lengths(4, 2048, 16384, seed=0), max_pos=16384)
+    elif args.workload == "ref_e2e":
+        import random
+        lens = ut.generate_array_with_avg(3584, 16, 4096, random.Random(0))
+        res = run_encoder(args, "reference end2end row: batch 16, max 4096, avg 3584 (python/benchmark/metrics/end2end:31)",
+                          768, 12, 3072, 12, "f16", lens)
+        res["vs_baseline"] = res["value"] / (16 / 0.09359)
+        res["baseline_note"] = "A100 fp16, 93.59 ms per 12-layer forward (other hardware)"
+    elif args.workload == "c2":
+        res = run_attention_only(args)
+    else:
+        res = run_membound_sweep(args)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -18,12 +18,16 @@
  *     python/util.py:37,45); NB = seq_blocks[B], T = 64 * NB tokens.
  *
  * Head-major packed layout (produced by rt_qkv_bias_split, consumed by
- * rt_bs_attention_fwd): for sequence s (n blocks, first global block g0) and head h
- * the 64x64 tiles of blocks 0..n-1 start at element (g0*H + h*n) * 4096; Q and K tiles
- * are row-major [token][d]; a V tile is stored transposed, [d][slot], where slot p of
- * every group of 16 holds token (p & ~15) | perm(p & 15), perm = {0,1,2,3,8,9,10,11,
- * 4,5,6,7,12,13,14,15} (the order in which a 32x32 MFMA accumulator hands P back as
- * the next MFMA's operand).  rt_unpack_v_tiles undoes it for inspection.
+ * rt_bs_attention_fwd): for sequence s (n blocks, first global block g0) and head h the
+ * 64x64 tiles of blocks 0..n-1 start at element (g0*H + h*n) * 4096.  A tile is stored in
+ * MFMA "fragment order": 8 fragments of 64 lanes x 8 elements; element e of lane l of
+ * fragment f is
+ *     Q, K :  tile[32*(f>>2) + (l&31)][16*(f&3) + 8*(l>>5) + e]         (row = token, col = d)
+ *     V    :  tile[token(16*(f&3) + 8*(l>>5) + e)][32*(f>>2) + (l&31)]  (transposed; token()
+ *             swaps bits 2 and 3 of the slot index, the order in which a 32x32 MFMA
+ *             accumulator hands P back as the next MFMA's operand)
+ * so that every operand load of the attention kernel is one coalesced 16-byte-per-lane
+ * request.  rt_unpack_head_tiles undoes the layout for inspection.
  */
 #ifndef RAPTOR_T_HIP_H
 #define RAPTOR_T_HIP_H
@@ -106,22 +110,25 @@ int rt_meta_partition_lpt(const int* seq_blocks, int batch, int heads, int n_wg,
 
 /* Replaces kernels::add_bias_and_transpose_kernel (layers/kernels/
  * add_bias_and_transpose.cu:212-233): qkv[T, 3*H*64] token-major + bias[3*H*64] ->
- * q (scaled by q_scale), k, vt in the head-major packed layout. */
+ * q (scaled by q_scale), k, vt in the head-major packed layout.  For rt_bs_attention_fwd
+ * q_scale must be log2(e)/sqrt(64): the attention kernel evaluates the softmax in base 2. */
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt,
                       const int* seq_blocks_dev, int batch, int total_blocks, int heads,
                       float q_scale, int dtype, void* stream);
 
-/* Inverse of the V-tile layout: vt (packed, transposed) -> v[T, H*64] token-major. */
-int rt_unpack_v_tiles(const void* vt, void* v, const int* seq_blocks_dev, int batch,
-                      int total_blocks, int heads, int dtype, void* stream);
+/* Inverse of the packed layout: packed tiles -> dst[T, H*64] token-major; transposed = 0
+ * for q / k, 1 for vt. */
+int rt_unpack_head_tiles(const void* packed, void* dst, const int* seq_blocks_dev, int batch,
+                         int total_blocks, int heads, int transposed, int dtype, void* stream);
 
 /* Replaces kernels::test_gemm_1 (layers/kernels/sparse_attention.cu:3192-3228) and the
  * two live kernels behind it (:2953-3190 balanced, :2111-2403 non balanced):
- * out[T, H*64] token-major = softmax over the listed key blocks of (q . k) @ v, the
- * scale already folded into q.  to_idx/to_pos: device CSR from rt_meta_build_to_index
+ * out[T, H*64] token-major = softmax over the listed key blocks of (q . k) @ v, evaluated
+ * as 2^(q.k) / sum 2^(q.k): the scale log2(e)/sqrt(d) is already folded into q.  to_idx/to_pos: device CSR from rt_meta_build_to_index
  * (plan_heads = 1 or heads).  If from_idx/from_pos are non-NULL the launch is
  * `n_wg` persistent workgroups each walking its slice of the LPT plan (balanced);
- * otherwise one workgroup per (head, from-block) unit. */
+ * otherwise the kernel enumerates the units itself (global rows first inside each
+ * (sequence, head) group, XCD-contiguous order). */
 int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out,
                         const int* seq_blocks_dev, int batch, int total_blocks, int heads,
                         const int* to_idx, const int* to_pos, int plan_heads,

@@ -20,7 +20,7 @@ RT_EINVAL, RT_ENOMEM, RT_EIO, RT_ENOSYS, RT_ECANCELED = -22, -12, -5, -38, -125
 EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
-    "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_v_tiles", "rt_bs_attention_fwd",
+    "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
@@ -54,7 +54,7 @@ def lib():
         L.rt_meta_block_costs.argtypes = [i32p, I, i32p, i64p]
         L.rt_meta_partition_lpt.argtypes = [i32p, I, I, I, i32p, i32p]
         L.rt_qkv_bias_split.argtypes = [vp, vp, vp, vp, vp, vp, I, I, I, F, I, vp]
-        L.rt_unpack_v_tiles.argtypes = [vp, vp, vp, I, I, I, I, vp]
+        L.rt_unpack_head_tiles.argtypes = [vp, vp, vp, I, I, I, I, I, vp]
         L.rt_bs_attention_fwd.argtypes = [vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
         L.rt_bias_residual_layernorm.argtypes = [vp, vp, vp, vp, vp, L64, I, F, I, vp]
         L.rt_bias_gelu.argtypes = [vp, vp, L64, I, I, vp]
@@ -163,10 +163,15 @@ def qkv_bias_split(qkv, bias, q, k, vt, seq_blocks_dev, heads, q_scale):
                                   heads, q_scale, _dtype_code(qkv), _stream()))
 
 
-def unpack_v_tiles(vt, v, seq_blocks_dev, heads):
+def unpack_head_tiles(packed, dst, seq_blocks_dev, heads, transposed):
     batch = seq_blocks_dev.numel() - 1
-    nb = v.shape[0] // 64
-    check(lib().rt_unpack_v_tiles(_dp(vt), _dp(v), _dp(seq_blocks_dev), batch, nb, heads, _dtype_code(v), _stream()))
+    nb = dst.shape[0] // 64
+    check(lib().rt_unpack_head_tiles(_dp(packed), _dp(dst), _dp(seq_blocks_dev), batch, nb, heads,
+                                     1 if transposed else 0, _dtype_code(dst), _stream()))
+
+
+LOG2E = 1.4426950408889634
+Q_SCALE = LOG2E / 8.0          # log2(e) / sqrt(64): what rt_bs_attention_fwd expects folded into q
 
 
 def bs_attention_fwd(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads,

@@ -1,30 +1,45 @@
 // Block-sparse (BigBird-pattern) attention forward for gfx950, d = 64, 64-token blocks.
 //
-// Work unit = (sequence, head, from-block): 64 queries against the key blocks its CSR
-// row lists (7/8 blocks for sparse rows, all n blocks for the two global rows).
+// Work unit = (sequence, head, from-block): 64 queries against the key blocks its CSR row
+// lists (7/8 blocks for a sparse row, all n blocks for the two global rows).
 //
-// Workgroup = 4 waves.  Wave w owns 32 queries (w & 1) and every second listed key block
-// (w >> 1): the two waves that share a key block share its K and V tiles in LDS, the two
-// key-block streams keep independent online-softmax states that are merged through LDS
-// once per unit.  Splitting the key list two ways halves the serial depth of the dense
-// rows and needs no exchange inside the loop.
+// One wave owns all 64 queries of a unit and streams K / V^T tiles straight from global
+// memory into MFMA operand registers: the QKV split kernel stores every 64x64 tile in
+// "fragment order" (8 fragments of 64 lanes x 16 bytes), so each operand load is one fully
+// coalesced 1 KiB request and the main loop needs no LDS and no barrier.  The next K tile
+// is requested as soon as the last QK^T product of the current tile has issued, the next
+// V^T tile after the last PV product: one register copy of each, latency covered by the
+// softmax and the other product.
+//
+//   sparse rows : one wave per unit, 4 units (adjacent from-blocks) per workgroup
+//   global rows : the 4 waves of a workgroup take every 4th key block of ONE unit and merge
+//                 their online-softmax states through LDS at the end
 //
 // MFMA formulation (v_mfma_f32_32x32x16_{f16,bf16}, fp32 accumulators):
-//   S^T[key][query] = K[key][:] . Q[query][:]      A = K tile from LDS, B = Q (registers)
-//   O^T[d][query]  += V^T[d][key] . P^T[key][query] A = V^T tile from LDS, B = P (registers)
-// Both products put the query on the accumulator's column (lane & 31), so row max, row
-// sum, the rescale factor and the final 1/sum are per-lane scalars, and the accumulator
-// registers of S^T are, after exp, exactly the B operand of the second product: P never
-// goes through LDS.  The V tile is stored transposed with its 64 key slots in accumulator
-// order by the QKV split kernel.
+//   S^T[key][query] = K[key][:] . Q[query][:]       A = K fragment,   B = Q fragment
+//   O^T[d][query]  += V^T[d][key] . P^T[key][query]  A = V^T fragment, B = P (registers)
+// Both products put the query on the accumulator column (lane & 31): max, sum and rescale
+// factors are per-lane scalars and the S^T accumulators, after exp2, are the B operand of
+// the second product, so P never leaves registers.
 //
-// LDS rows are padded from 128 to 144 bytes so that the 16-byte operand reads of 16
-// consecutive rows fall in distinct banks.
+// Softmax is evaluated in base 2 (q arrives pre-multiplied by log2(e)/sqrt(d)).  The S^T
+// accumulator starts at minus the row's reference maximum, so the MFMA result feeds exp2
+// directly; the reference is only moved (and O, l rescaled) when a new score exceeds it
+// by more than 2^6, which keeps every P value below 64 and makes the rescale a rare,
+// wave-uniform branch.
+//
+// Launch without a plan: workgroups enumerate (sequence, head) groups in order, global rows
+// first inside each group, and consecutive workgroup ids are remapped so that each XCD
+// (one L2 per XCD, workgroups are dealt round-robin to the 8 XCDs) walks a contiguous
+// range of groups: the K/V tiles of a (sequence, head) stay in one L2.
+// Launch with an LPT plan: n_wg persistent workgroups walk their unit lists.
 //
 // Replaces, from the reference: layers/kernels/sparse_attention.cu:2953-3190 (balanced,
 // persistent workgroups over the LPT plan), :2111-2403 (one workgroup per unit) and the
 // dispatcher :3192-3228.
 #include <hip/hip_runtime.h>
+
+#include <cstdlib>
 
 #include "rt_common.h"
 
@@ -34,202 +49,528 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+
+__device__ inline uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
+}
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
   typedef f16x8 v8;
   typedef f16x4 v4;
   __device__ static f32x16 run(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  // a[0..7] = p[0..7] rounded to T; returns the fp32 sum of the ROUNDED values (what PV multiplies)
+  __device__ static float pack(const float* p, v8& out) {
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      f16x2 h = {static_cast<_Float16>(p[e]), static_cast<_Float16>(p[e + 1])};
+      out[e] = h[0];
+      out[e + 1] = h[1];
+      s = __builtin_amdgcn_fdot2(h, f16x2{1, 1}, s, false);
+    }
+    return s;
+  }
+  // positive halves order like unsigned 16-bit integers: running packed maximum of the bit patterns
+  __device__ static uint32_t max_bits(const v8& p, uint32_t acc) {
+    const u32x4 w = __builtin_bit_cast(u32x4, p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = pk_max_u16(acc, w[i]);
+    return acc;
+  }
+  __device__ static bool over_threshold(uint32_t top) {      // 64.0 in fp16 is 0x5400
+    return (top & 0xffffu) > 0x5400u || (top >> 16) > 0x5400u;
+  }
 };
 template <> struct Mma<__bf16> {
   typedef bf16x8 v8;
   typedef bf16x4 v4;
   __device__ static f32x16 run(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  __device__ static float pack(const float* p, v8& out) {
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      out[e] = static_cast<__bf16>(p[e]);
+      s += static_cast<float>(out[e]);
+    }
+    return s;
+  }
+  __device__ static uint32_t max_bits(const v8& p, uint32_t acc) {
+    const u32x4 w = __builtin_bit_cast(u32x4, p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = pk_max_u16(acc, w[i]);
+    return acc;
+  }
+  __device__ static bool over_threshold(uint32_t top) {      // 64.0 in bf16 is 0x4280
+    return (top & 0xffffu) > 0x4280u || (top >> 16) > 0x4280u;
+  }
 };
 
-constexpr int ROW = 72;                 // padded LDS row, in elements (144 bytes)
-constexpr int TILE = 64 * ROW;          // one K or V^T tile in LDS
-constexpr float LOG2E = 1.4426950408889634f;
+// A row's reference maximum only moves when some P = 2^(score - reference) would exceed 2^6
+// (tested on the packed 16-bit P values; see over_threshold).
 
-__device__ inline int find_seq_by_unit(const int* __restrict__ seq_blocks, int batch, int heads, int unit) {
-  int lo = 0, hi = batch;               // seq_blocks[lo]*heads <= unit < seq_blocks[hi]*heads
+// Online-softmax state of one wave for its 64 queries: O^T as [d tile][query tile].
+struct State {
+  f32x16 o[2][2];
+  float m[2], l[2];      // per query tile: reference maximum (log2 units), partial row sum
+};
+
+__device__ inline void state_init(State& st) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) st.o[t][nt][e] = 0.f;
+  st.m[0] = st.m[1] = -INFINITY;
+  st.l[0] = st.l[1] = 0.f;
+}
+
+template <typename T>
+__device__ inline void load_tile(const T* __restrict__ tile, int lane, typename Mma<T>::v8 (&f)[8]) {
+  typedef typename Mma<T>::v8 v8;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = *reinterpret_cast<const v8*>(tile + i * 512 + lane * 8);
+}
+
+// Streams key blocks row[first], row[first + step], ... of one (sequence, head) through the
+// state.  kbase / vbase point at block 0 of that (sequence, head); n = blocks in the sequence.
+// The row's block ids are fetched 64 at a time into one register (lane j holds entry j) and
+// handed out with v_readlane: one memory round trip per unit instead of one per key block.
+template <typename T>
+__device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __restrict__ vbase,
+                                    const int* __restrict__ row, int first, int step, int cnt, int n, int lane,
+                                    const typename Mma<T>::v8 (&qf)[2][4], State& st) {
+  typedef typename Mma<T>::v8 v8;
+  if (first >= cnt) return;
+  int chunk = first >> 6;
+  int ids = (chunk * 64 + lane < cnt) ? row[chunk * 64 + lane] : 0;
+  auto block_of = [&](int j) {                        // j is wave-uniform
+    if ((j >> 6) != chunk) {
+      chunk = j >> 6;
+      ids = (chunk * 64 + lane < cnt) ? row[chunk * 64 + lane] : 0;
+    }
+    const int b = __builtin_amdgcn_readlane(ids, j & 63);
+    return b < 0 ? 0 : (b >= n ? n - 1 : b);
+  };
+  v8 kf[8], vf[8];
+  {
+    const int b = block_of(first);
+    load_tile<T>(kbase + int64_t(b) * 4096, lane, kf);
+    load_tile<T>(vbase + int64_t(b) * 4096, lane, vf);
+  }
+  bool fresh = true;                                  // no reference maximum yet
+  for (int j = first; j < cnt; j += step) {
+    const int jn = j + step;
+    const bool more = jn < cnt;
+    // the last iteration re-requests its own tile: loads stay unconditional, so they keep
+    // their place in the instruction stream (a branch would sink them next to their use)
+    const int bn = block_of(more ? jn : j);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      f32x16 sc[2];
+      v8 pb[4];
+      float psum;
+      auto scores = [&](float init) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) sc[t][e] = init;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+#ifndef RT_X_NOQK
+            sc[t] = Mma<T>::run(kf[t * 4 + c], qf[nt][c], sc[t]);
+#else
+            sc[t][c] += float(kf[t * 4 + c][0]) + float(qf[nt][c][0]);
+#endif
+          }
+        }
+      };
+      // exp2 of the (already shifted) scores -> P as the B operand of the second product:
+      // step s takes accumulator registers 8*(s&1)..+7 of key tile s>>1.  Returns true when
+      // some P exceeds 2^RESCALE_THRESHOLD (or is not finite).
+      auto exponentiate = [&]() {
+        float part[4];
+        uint32_t top = 0;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          float p8[8];
+#pragma unroll
+#ifndef RT_X_NOEXP
+          for (int e = 0; e < 8; ++e) p8[e] = __builtin_amdgcn_exp2f(sc[s >> 1][8 * (s & 1) + e]);
+#else
+          for (int e = 0; e < 8; ++e) p8[e] = sc[s >> 1][8 * (s & 1) + e];
+#endif
+#ifndef RT_X_NOSUM
+          part[s] = Mma<T>::pack(p8, pb[s]);
+          top = Mma<T>::max_bits(pb[s], top);
+#else
+          for (int e = 0; e < 8; ++e) pb[s][e] = static_cast<T>(p8[e]);
+          part[s] = 0.f;
+#endif
+        }
+        psum = (part[0] + part[1]) + (part[2] + part[3]);
+        return Mma<T>::over_threshold(top);
+      };
+      bool redo = fresh;
+      if (!fresh) {
+        scores(-st.m[nt]);
+        redo = __any(exponentiate());
+      }
+      if (redo) {
+        // rare (always on the first tile): find the true maximum and move the reference there
+        scores(0.f);
+        float mx = sc[0][0];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[t][e]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fresh ? mx : fmaxf(mx, st.m[nt]);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) sc[t][e] -= m_new;
+        if (!fresh) {
+          const float alpha = __builtin_amdgcn_exp2f(st.m[nt] - m_new);
+          st.l[nt] *= alpha;
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) st.o[t][nt][e] *= alpha;
+        }
+        st.m[nt] = m_new;
+        (void)exponentiate();
+      }
+      // the K fragments are dead once the second query tile's scores are final
+#ifndef RT_X_NOLOAD
+      if (nt == 1) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_tile<T>(kbase + int64_t(bn) * 4096, lane, kf);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#endif
+      st.l[nt] += psum;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+#ifndef RT_X_NOPV
+        for (int s = 0; s < 4; ++s) st.o[t][nt] = Mma<T>::run(vf[t * 4 + s], pb[s], st.o[t][nt]);
+#else
+        for (int s = 0; s < 4; ++s) st.o[t][nt][s] += float(vf[t * 4 + s][0]) + float(pb[s][0]) + float(pb[s][7]);
+#endif
+    }
+    fresh = false;
+#ifndef RT_X_NOLOAD
+    __builtin_amdgcn_sched_barrier(0);
+    load_tile<T>(vbase + int64_t(bn) * 4096, lane, vf);
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+  }
+}
+
+// Writes the wave's 64x64 output tile, O^T[d = 32t + 8*(e>>2) + 4*(lane>>5) + (e&3)]
+// [query 32nt + (lane&31)] * w, to out[token][h*64 + d].  The tile is transposed through a
+// wave-private LDS region (64 rows of 64 + 4 elements) so that every global store covers
+// whole 128-byte row segments: 8 lanes x 16 bytes per row.
+constexpr int STAGE_ROW = 68;                       // elements; 136 bytes keeps ds_write_b64 conflict free
+constexpr int STAGE_BYTES = 64 * STAGE_ROW * 2;     // 8704 bytes per wave
+
+template <typename T>
+__device__ inline void store_output(T* __restrict__ out_unit, int64_t row_stride, int lane, const State& st,
+                                    const float (&w)[2], T* __restrict__ stage) {
+  typedef typename Mma<T>::v4 v4;
+  typedef typename Mma<T>::v8 v8;
+  const int l32 = lane & 31, hi = lane >> 5;
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    T* sp = stage + (32 * nt + l32) * STAGE_ROW + 4 * hi;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        v4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = static_cast<T>(st.o[t][nt][4 * c4 + e] * w[nt]);
+        *reinterpret_cast<v4*>(sp + 32 * t + 8 * c4) = r;
+      }
+  }
+  __builtin_amdgcn_wave_barrier();                  // same wave wrote it: LDS is in order per wave
+  const int r8 = lane >> 3, c8 = (lane & 7) * 8;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int row = 8 * it + r8;
+    const v4* src = reinterpret_cast<const v4*>(stage + row * STAGE_ROW + c8);   // rows are 8-byte aligned
+    const v4 lo = src[0], up = src[1];
+    const v8 v = {lo[0], lo[1], lo[2], lo[3], up[0], up[1], up[2], up[3]};
+    *reinterpret_cast<v8*>(out_unit + int64_t(row) * row_stride + c8) = v;
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+struct Unit {
+  int h, i, n, g0;
+};
+
+template <typename T> struct Args {
+  const T* q; const T* k; const T* vt; T* out;
+  const int* seq_blocks; int batch, heads, nb_total;
+  const int* to_idx; const int* to_pos; int plan_heads;
+  const int* from_idx; const int* from_pos;
+};
+
+constexpr int MAX_BATCH = 1024;         // sequences per launch (geometry is kept in LDS)
+
+// Geometry of the batch in LDS: sb = prefix blocks, gl / bu = prefix counts of the plan-free
+// launch's global items and bundles (per sequence, times heads).
+struct Geometry {
+  int sb[MAX_BATCH + 1];
+  int gl[MAX_BATCH + 1];
+  int bu[MAX_BATCH + 1];
+};
+
+__device__ inline int upper_seq(const int* __restrict__ prefix, int batch, int x) {
+  int lo = 0, hi = batch;               // prefix[lo] <= x < prefix[hi]
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
-    if (seq_blocks[mid] * heads <= unit) lo = mid; else hi = mid;
+    if (prefix[mid] <= x) lo = mid; else hi = mid;
   }
   return lo;
 }
 
+__device__ inline bool is_global_row(const Unit& u) { return u.n >= RT_MIN_SPARSE_BLOCKS && (u.i == 0 || u.i == u.n - 1); }
+
 template <typename T>
-__global__ __launch_bounds__(256, 2) void bs_attention_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt, T* __restrict__ out,
-    const int* __restrict__ seq_blocks, int batch, int heads, int nb_total, const int* __restrict__ to_idx,
-    const int* __restrict__ to_pos, int plan_heads, const int* __restrict__ from_idx,
-    const int* __restrict__ from_pos) {
+__device__ inline void load_q(const Args<T>& a, const Unit& u, int lane, typename Mma<T>::v8 (&qf)[2][4]) {
   typedef typename Mma<T>::v8 v8;
-  typedef typename Mma<T>::v4 v4;
-  __shared__ __attribute__((aligned(16))) T smem[2 * 2 * TILE];     // [key stream][K | V^T]
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int qh = wave & 1, ks = wave >> 1;           // query half, key stream
-  const int l32 = lane & 31, hi = lane >> 5;
-  const int ptid = tid & 127;                        // thread index inside the key stream's pair of waves
-  T* lds_k = smem + ks * 2 * TILE;
-  T* lds_v = lds_k + TILE;
-
-  int u_begin, u_end;
-  if (from_pos) { u_begin = from_pos[blockIdx.x]; u_end = from_pos[blockIdx.x + 1]; }
-  else { u_begin = blockIdx.x; u_end = u_begin + 1; }
-  const int n_units = nb_total * heads;
-
-  for (int ui = u_begin; ui < u_end; ++ui) {
-    const int unit = from_idx ? from_idx[ui] : ui;
-    if (unit < 0 || unit >= n_units) continue;       // uniform over the workgroup
-    const int s = find_seq_by_unit(seq_blocks, batch, heads, unit);
-    const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
-    const int rem = unit - g0 * heads;
-    const int h = rem / n, i = rem - h * n;
-    const int64_t base = (int64_t(g0) * heads + int64_t(h) * n) * 4096;
-    const int row = (plan_heads > 1 ? h : 0) * nb_total + g0 + i;
-    const int p0 = to_pos[row];
-    const int cnt = to_pos[row + 1] - p0;
-    const int iters = (cnt + 1) >> 1;
-
-    // Q fragments: B operand of S^T, Q[query = 32*qh + l32][d = 16*c + 8*hi .. +7]
-    v8 qf[4];
-    {
-      const T* qp = q + base + int64_t(i) * 4096 + (32 * qh + l32) * 64 + 8 * hi;
+  const T* qt = a.q + (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n + u.i) * 4096;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) qf[c] = *reinterpret_cast<const v8*>(qp + 16 * c);
-    }
-    f32x16 o_acc[2];
+  for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) qf[nt][c] = *reinterpret_cast<const v8*>(qt + (nt * 4 + c) * 512 + lane * 8);
+}
+
+// One wave, one unit, all of its key blocks.
+template <typename T>
+__device__ inline void run_solo(const Args<T>& a, const Unit& u, int lane, T* stage) {
+  typename Mma<T>::v8 qf[2][4];
+  const int row = (a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i;
+  const int p0 = __builtin_amdgcn_readfirstlane(a.to_pos[row]);
+  const int cnt = __builtin_amdgcn_readfirstlane(a.to_pos[row + 1]) - p0;
+  load_q<T>(a, u, lane, qf);
+  const int64_t base = (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n) * 4096;
+  State st;
+  state_init(st);
+  stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, lane, qf, st);
+#ifdef RT_X_REPEAT
+  for (int rep = 1; rep < RT_X_REPEAT; ++rep) stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, lane, qf, st);
+#endif
+  float w[2];
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) {
+    const float l = st.l[nt] + __shfl_xor(st.l[nt], 32, 64);
+    w[nt] = 1.0f / fmaxf(l, 1e-30f);
+  }
+  const int64_t stride = int64_t(a.heads) * 64;
+  store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w, stage);
+}
+
+// Four waves, one unit: wave w streams key blocks w, w+4, ...; tree merge through LDS.
+template <typename T>
+__device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int wave, float* park) {
+  typename Mma<T>::v8 qf[2][4];
+  const int row = (a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i;
+  const int p0 = __builtin_amdgcn_readfirstlane(a.to_pos[row]);
+  const int cnt = __builtin_amdgcn_readfirstlane(a.to_pos[row + 1]) - p0;
+  load_q<T>(a, u, lane, qf);
+  const int64_t base = (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n) * 4096;
+  State st;
+  state_init(st);
+  stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, lane, qf, st);
+#ifdef RT_X_REPEAT
+  for (int rep = 1; rep < RT_X_REPEAT; ++rep) stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, lane, qf, st);
+#endif
+#pragma unroll
+  for (int nt = 0; nt < 2; ++nt) st.l[nt] += __shfl_xor(st.l[nt], 32, 64);
+
+  auto dump = [&](float* slot) {
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o_acc[t][e] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-
-    v8 pk[4], pv[4];                                  // this thread's 64 bytes of the next K and V^T tiles
-    auto gload = [&](int j) {
-      int blk = to_idx[p0 + j];
-      blk = blk < 0 ? 0 : (blk >= n ? n - 1 : blk);
-      const T* kp = k + base + int64_t(blk) * 4096;
-      const T* vp = vt + base + int64_t(blk) * 4096;
+      for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        pk[c] = *reinterpret_cast<const v8*>(kp + (ptid + 128 * c) * 8);
-        pv[c] = *reinterpret_cast<const v8*>(vp + (ptid + 128 * c) * 8);
-      }
-    };
-    if (ks < cnt) gload(ks);
-
-    for (int it = 0; it < iters; ++it) {
-      const int j = 2 * it + ks;
-      const bool valid = j < cnt;
-      __syncthreads();                                // every wave is done reading the previous tiles
-      if (valid) {
+        for (int e = 0; e < 16; ++e) slot[((t * 2 + nt) * 16 + e) * 64 + lane] = st.o[t][nt][e];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int chunk = ptid + 128 * c;
-          const int off = (chunk >> 3) * ROW + (chunk & 7) * 8;
-          *reinterpret_cast<v8*>(lds_k + off) = pk[c];
-          *reinterpret_cast<v8*>(lds_v + off) = pv[c];
-        }
-      }
-      __syncthreads();                                // tiles visible
-      if (j + 2 < cnt) gload(j + 2);                  // in flight during the MFMAs below
-      if (!valid) continue;
-
-      f32x16 sc[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) sc[t][e] = 0.f;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const v8 a = *reinterpret_cast<const v8*>(lds_k + (32 * t + l32) * ROW + 16 * c + 8 * hi);
-          sc[t] = Mma<T>::run(a, qf[c], sc[t]);
-        }
-      }
-      // online softmax; the lane holds 32 of its query's 64 scores, lane ^ 32 the others
-      float mx = sc[0][0];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[t][e]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
-      const float mb = m_new * LOG2E;
-      float psum = 0.f;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          sc[t][e] = __builtin_amdgcn_exp2f(sc[t][e] * LOG2E - mb);
-          psum += sc[t][e];
-        }
-      l_run = l_run * alpha + psum;
-      m_run = m_new;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
-      // P as the B operand: step st takes accumulator registers 8*(st&1)..+7 of tile st>>1
-      v8 pb[4];
-#pragma unroll
-      for (int st = 0; st < 4; ++st)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pb[st][e] = static_cast<T>(sc[st >> 1][8 * (st & 1) + e]);
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int st = 0; st < 4; ++st) {
-          const v8 a = *reinterpret_cast<const v8*>(lds_v + (32 * t + l32) * ROW + 16 * st + 8 * hi);
-          o_acc[t] = Mma<T>::run(a, pb[st], o_acc[t]);
-        }
+    for (int nt = 0; nt < 2; ++nt) {
+      slot[(64 + nt) * 64 + lane] = st.m[nt];
+      slot[(66 + nt) * 64 + lane] = st.l[nt];
     }
-
-    // merge the two key streams: stream 1 parks (O, m, l) in LDS, stream 0 combines and stores
-    l_run += __shfl_xor(l_run, 32, 64);
-    __syncthreads();                                  // all tile reads finished before LDS is reused
-    float* park = reinterpret_cast<float*>(smem) + qh * (34 * 64);
-    if (ks == 1) {
+  };
+  auto absorb = [&](const float* slot) {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const float m1 = slot[(64 + nt) * 64 + lane], l1 = slot[(66 + nt) * 64 + lane];
+      const float mt = fmaxf(fmaxf(st.m[nt], m1), -1e30f);        // finite even if both are empty
+      const float a0 = __builtin_amdgcn_exp2f(st.m[nt] - mt), a1 = __builtin_amdgcn_exp2f(m1 - mt);
+      st.m[nt] = mt;
+      st.l[nt] = st.l[nt] * a0 + l1 * a1;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) park[(16 * t + e) * 64 + lane] = o_acc[t][e];
-      park[32 * 64 + lane] = m_run;
-      park[33 * 64 + lane] = l_run;
+        for (int e = 0; e < 16; ++e)
+          st.o[t][nt][e] = st.o[t][nt][e] * a0 + slot[((t * 2 + nt) * 16 + e) * 64 + lane] * a1;
     }
-    __syncthreads();
-    if (ks == 0) {
-      const float m1 = park[32 * 64 + lane], l1 = park[33 * 64 + lane];
-      const float m_tot = fmaxf(fmaxf(m_run, m1), -1e30f);      // finite even for an empty row
-      const float a0 = __builtin_amdgcn_exp2f((m_run - m_tot) * LOG2E);
-      const float a1 = __builtin_amdgcn_exp2f((m1 - m_tot) * LOG2E);
-      const float inv = 1.0f / fmaxf(l_run * a0 + l1 * a1, 1e-30f);
-      const float w0 = a0 * inv, w1 = a1 * inv;
-      // O^T[d = 32*t + 8*(e>>2) + 4*hi + (e&3)][query l32] -> out[token][h*64 + d]
-      T* op = out + (int64_t(g0 + i) * 64 + 32 * qh + l32) * (int64_t(heads) * 64) + h * 64 + 4 * hi;
+  };
+  __syncthreads();                                    // the park is free (previous item is over)
+  if (wave >= 2) dump(park + (wave - 2) * (68 * 64));
+  __syncthreads();
+  if (wave < 2) absorb(park + wave * (68 * 64));
+  __syncthreads();
+  if (wave == 1) dump(park);
+  __syncthreads();
+  if (wave == 0) {
+    absorb(park);
+    float w[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) {
-          v4 r;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int v = 4 * c4 + e;
-            r[e] = static_cast<T>(o_acc[t][v] * w0 + park[(16 * t + v) * 64 + lane] * w1);
-          }
-          *reinterpret_cast<v4*>(op + 32 * t + 8 * c4) = r;
-        }
-    }
+    for (int nt = 0; nt < 2; ++nt) w[nt] = 1.0f / fmaxf(st.l[nt], 1e-30f);
+    const int64_t stride = int64_t(a.heads) * 64;
+    // slot 1 of the park was consumed before the third barrier: reuse it as the staging tile
+    store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w,
+                    reinterpret_cast<T*>(park + 68 * 64));
   }
+  __syncthreads();                                    // the park is free again (solo waves stage their output in it)
+}
+
+__device__ __host__ inline int bundles_per_head(int n) {
+  return n >= RT_MIN_SPARSE_BLOCKS ? (n - 2 + 3) / 4 : (n + 3) / 4;
+}
+
+// Persistent workgroups (two per CU).
+//
+// With an LPT plan (from_idx / from_pos): workgroup c walks its slice of the plan; global rows
+// are shared by its four waves, runs of up to four other units go one per wave.
+//
+// Without a plan the kernel makes its own schedule.  Two kinds of items:
+//   global item : one global row (first or last block of a sequence of >= 12 blocks), 4 waves
+//   bundle      : up to 4 consecutive other rows of one (sequence, head), one per wave
+// numbered sequence-major, then head.  Workgroups are dealt to the 8 XCDs round-robin by the
+// hardware; the workgroups of XCD x share the x-th eighth of the global items FIRST (they are
+// the long ones) and then the x-th eighth of the bundles, which covers (nearly) the same
+// (sequence, head) groups, so a group's K/V tiles stay in one L2.
+template <typename T>
+__global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
+  // 34816 bytes: two parked wave states for the global-row merge, or four output staging tiles
+  __shared__ __attribute__((aligned(16))) float park[2 * 68 * 64];
+  __shared__ Geometry geo;
+  static_assert(4 * STAGE_BYTES <= sizeof(float) * 2 * 68 * 64, "staging tiles must fit in the park");
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  T* stage = reinterpret_cast<T*>(reinterpret_cast<char*>(park) + wave * STAGE_BYTES);
+
+  for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int g = 0, b = 0;
+    for (int s = 0; s < a.batch; ++s) {
+      geo.gl[s] = g;
+      geo.bu[s] = b;
+      const int n = geo.sb[s + 1] - geo.sb[s];
+      g += (n >= RT_MIN_SPARSE_BLOCKS ? 2 : 0) * a.heads;
+      b += bundles_per_head(n) * a.heads;
+    }
+    geo.gl[a.batch] = g;
+    geo.bu[a.batch] = b;
+  }
+  __syncthreads();
+
+  auto unit_of_flat = [&](int unit) {               // flat id = blk + head * n_s + seq_start * heads
+    int lo = 0, hi = a.batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (geo.sb[mid] * a.heads <= unit) lo = mid; else hi = mid;
+    }
+    Unit u;
+    u.g0 = geo.sb[lo];
+    u.n = geo.sb[lo + 1] - u.g0;
+    const int rem = unit - u.g0 * a.heads;
+    u.h = rem / u.n;
+    u.i = rem - u.h * u.n;
+    return u;
+  };
+
+  if (a.from_pos) {
+    int p = a.from_pos[blockIdx.x];
+    const int end = a.from_pos[blockIdx.x + 1];
+    const int n_units = a.nb_total * a.heads;
+    while (p < end) {
+      // the next four plan entries in one round trip
+      const int mine_id = (p + wave < end) ? a.from_idx[p + wave] : -1;
+      int ids4[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) ids4[w] = (p + w < end) ? a.from_idx[p + w] : -1;
+      if (ids4[0] < 0 || ids4[0] >= n_units) { ++p; continue; }
+      const Unit first = unit_of_flat(ids4[0]);
+      if (is_global_row(first)) {
+        run_split4<T>(a, first, lane, wave, park);
+        ++p;
+        continue;
+      }
+      int run = 1;
+      while (run < 4 && ids4[run] >= 0 && ids4[run] < n_units && !is_global_row(unit_of_flat(ids4[run]))) ++run;
+      if (wave < run) run_solo<T>(a, unit_of_flat(mine_id), lane, stage);
+      p += run;
+    }
+    return;
+  }
+
+  const int n_glob = geo.gl[a.batch], n_bund = geo.bu[a.batch];
+  const int x = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
+  const int g_lo = int(int64_t(n_glob) * x / 8), g_cnt = int(int64_t(n_glob) * (x + 1) / 8) - g_lo;
+  const int b_lo = int(int64_t(n_bund) * x / 8), b_cnt = int(int64_t(n_bund) * (x + 1) / 8) - b_lo;
+  for (int k = blockIdx.x >> 3; k < g_cnt + b_cnt; k += per_xcd) {
+    Unit u;
+    if (k < g_cnt) {
+      const int item = g_lo + k;
+      const int s = upper_seq(geo.gl, a.batch, item);
+      const int rem = item - geo.gl[s];
+      u.g0 = geo.sb[s];
+      u.n = geo.sb[s + 1] - u.g0;
+      u.h = rem >> 1;
+      u.i = (rem & 1) ? u.n - 1 : 0;
+      run_split4<T>(a, u, lane, wave, park);
+      continue;
+    }
+    const int item = b_lo + (k - g_cnt);
+    const int s = upper_seq(geo.bu, a.batch, item);
+    const int rem = item - geo.bu[s];
+    u.g0 = geo.sb[s];
+    u.n = geo.sb[s + 1] - u.g0;
+    const int per_head = bundles_per_head(u.n);
+    u.h = rem / per_head;
+    const int bundle = rem - u.h * per_head;
+    const bool sparse = u.n >= RT_MIN_SPARSE_BLOCKS;
+    u.i = (sparse ? 1 : 0) + 4 * bundle + wave;
+    if (u.i <= (sparse ? u.n - 2 : u.n - 1)) run_solo<T>(a, u, lane, stage);
+  }
+}
+
+// Two persistent workgroups per CU, a multiple of 8 so that every XCD gets the same number.
+unsigned plan_free_workgroups() {
+#ifdef RT_X_ENVWGS
+  if (const char* e = getenv("RT_X_WGS")) return unsigned(atoi(e));
+#endif
+  static unsigned cached = 0;
+  if (cached == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    cached = unsigned((2 * cus + 7) / 8 * 8);
+  }
+  return cached;
 }
 
 }  // namespace
@@ -244,6 +585,7 @@ extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt,
   RT_REQUIRE(plan_heads == 1 || plan_heads == heads, RT_EINVAL, "plan_heads=%d must be 1 or heads=%d", plan_heads, heads);
   RT_REQUIRE((from_idx == nullptr) == (from_pos == nullptr), RT_EINVAL, "from_idx and from_pos go together");
   RT_REQUIRE(int64_t(total_blocks) * heads < (int64_t(1) << 31), RT_EINVAL, "too many units");
+  RT_REQUIRE(batch <= MAX_BATCH, RT_EINVAL, "at most %d sequences per launch, got %d", MAX_BATCH, batch);
   RT_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(vt) |
                reinterpret_cast<uintptr_t>(out)) & 15u) == 0, RT_EINVAL, "q, k, vt, out must be 16-byte aligned");
   if (dtype == RT_F32) return rt::fail(RT_ENOSYS, "block-sparse attention runs in fp16 or bf16 (fp32 accumulation)");
@@ -253,17 +595,18 @@ extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt,
     RT_REQUIRE(n_wg >= 1, RT_EINVAL, "balanced launch needs n_wg >= 1, got %d", n_wg);
     grid = unsigned(n_wg);
   } else {
-    grid = unsigned(total_blocks) * unsigned(heads);
+    grid = plan_free_workgroups();
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == RT_F16)
-    hipLaunchKernelGGL(bs_attention_kernel<_Float16>, dim3(grid), dim3(256), 0, st, (const _Float16*)q, (const _Float16*)k,
-                       (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch, heads, total_blocks, to_idx, to_pos,
-                       plan_heads, from_idx, from_pos);
-  else
-    hipLaunchKernelGGL(bs_attention_kernel<__bf16>, dim3(grid), dim3(256), 0, st, (const __bf16*)q, (const __bf16*)k,
-                       (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads, total_blocks, to_idx, to_pos,
-                       plan_heads, from_idx, from_pos);
+  if (dtype == RT_F16) {
+    Args<_Float16> a{(const _Float16*)q, (const _Float16*)k, (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch,
+                     heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos};
+    hipLaunchKernelGGL(bs_attention_kernel<_Float16>, dim3(grid), dim3(256), 0, st, a);
+  } else {
+    Args<__bf16> a{(const __bf16*)q, (const __bf16*)k, (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads,
+                   total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos};
+    hipLaunchKernelGGL(bs_attention_kernel<__bf16>, dim3(grid), dim3(256), 0, st, a);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "bs_attention launch failed: %s", hipGetErrorString(e));
   return RT_OK;

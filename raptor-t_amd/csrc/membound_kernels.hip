@@ -229,8 +229,14 @@ __global__ __launch_bounds__(256) void bias_gelu_kernel(T* __restrict__ out, con
 }
 
 // ---- QKV bias + scale + head split --------------------------------------------------------
-// Workgroup (g, h): global block g, head h.  Q and K tiles are copied row-major; the V
-// tile goes through LDS and is written transposed with the MFMA slot order.
+// Workgroup (g, h): global block g, head h.  The three 64x64 tiles are staged in LDS (bias
+// and scale applied) and written out in MFMA "fragment order": a tile is 8 fragments of
+// 64 lanes x 8 elements, element e of lane l of fragment f being
+//     Q, K :  tile[32*(f>>2) + (l&31)][16*(f&3) + 8*(l>>5) + e]        (row = token, col = d)
+//     V    :  tile[token(16*(f&3) + 8*(l>>5) + e)][32*(f>>2) + (l&31)] (transposed; token()
+//             swaps bits 2 and 3 of the slot index: the order in which a 32x32 accumulator
+//             hands P back as an MFMA operand)
+// so the attention kernel loads each operand with one coalesced 16-byte-per-lane request.
 __device__ inline int find_seq(const int* __restrict__ seq_blocks, int batch, int g) {
   int lo = 0, hi = batch;                   // seq_blocks[lo] <= g < seq_blocks[hi]
   while (hi - lo > 1) {
@@ -245,6 +251,12 @@ __device__ inline int slot_token(int p) {   // token held by slot p of a transpo
   return (p & ~15) | ((e & 3) | ((e & 4) << 1) | ((e & 8) >> 1));
 }
 
+template <typename T> __device__ inline void store8(T* p, const float* x) {
+  constexpr int N = Vec<T>::N;
+#pragma unroll
+  for (int i = 0; i < 8; i += N) Vec<T>::store(p + i, x + i);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
                                                              T* __restrict__ q, T* __restrict__ k,
@@ -252,53 +264,59 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
                                                              int batch, int heads, float q_scale) {
   constexpr int N = Vec<T>::N;              // elements per 16 bytes
   constexpr int CPR = 64 / N;               // 16-byte chunks per 64-wide row
-  __shared__ float vtile[64][65];
+  __shared__ float tile[3][64][65];
   const int g = blockIdx.x, h = blockIdx.y;
   const int s = find_seq(seq_blocks, batch, g);
   const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
-  const int64_t tile = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
+  const int64_t base = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
   const int dm = heads * 64;
   const T* src = qkv + int64_t(g) * 64 * (3 * dm) + h * 64;
   for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
     const int row = c / CPR, col = (c % CPR) * N;
-    float x[N], b[N];
-    Vec<T>::load(src + int64_t(row) * 3 * dm + col, x);
-    Vec<T>::load(bias + h * 64 + col, b);
 #pragma unroll
-    for (int i = 0; i < N; ++i) x[i] = (x[i] + b[i]) * q_scale;
-    Vec<T>::store(q + tile + row * 64 + col, x);
-    Vec<T>::load(src + int64_t(row) * 3 * dm + dm + col, x);
-    Vec<T>::load(bias + dm + h * 64 + col, b);
+    for (int m = 0; m < 3; ++m) {
+      float x[N], b[N];
+      Vec<T>::load(src + int64_t(row) * 3 * dm + m * dm + col, x);
+      Vec<T>::load(bias + m * dm + h * 64 + col, b);
+      const float sc = m == 0 ? q_scale : 1.0f;
 #pragma unroll
-    for (int i = 0; i < N; ++i) x[i] += b[i];
-    Vec<T>::store(k + tile + row * 64 + col, x);
-    Vec<T>::load(src + int64_t(row) * 3 * dm + 2 * dm + col, x);
-    Vec<T>::load(bias + 2 * dm + h * 64 + col, b);
-#pragma unroll
-    for (int i = 0; i < N; ++i) vtile[row][col + i] = x[i] + b[i];
+      for (int i = 0; i < N; ++i) tile[m][row][col + i] = (x[i] + b[i]) * sc;
+    }
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
-    const int d = c / CPR, p0 = (c % CPR) * N;
-    float x[N];
+  for (int c = threadIdx.x; c < 512; c += 256) {
+    const int f = c >> 6, l = c & 63;
+    const int r32 = 32 * (f >> 2) + (l & 31), c8 = 16 * (f & 3) + 8 * (l >> 5);
+    float x[8];
 #pragma unroll
-    for (int i = 0; i < N; ++i) x[i] = vtile[slot_token(p0 + i)][d];
-    Vec<T>::store(vt + tile + d * 64 + p0, x);
+    for (int e = 0; e < 8; ++e) x[e] = tile[0][r32][c8 + e];
+    store8<T>(q + base + c * 8, x);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = tile[1][r32][c8 + e];
+    store8<T>(k + base + c * 8, x);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = tile[2][slot_token(c8 + e)][r32];
+    store8<T>(vt + base + c * 8, x);
   }
 }
 
+// Inverse of the fragment order for inspection: packed tiles -> token-major [T, H*64].
+// transposed = 0 for Q / K tiles, 1 for V tiles.
 template <typename T>
-__global__ __launch_bounds__(256) void unpack_v_tiles_kernel(const T* __restrict__ vt, T* __restrict__ v,
-                                                             const int* __restrict__ seq_blocks, int batch,
-                                                             int heads) {
+__global__ __launch_bounds__(256) void unpack_head_tiles_kernel(const T* __restrict__ packed, T* __restrict__ dst,
+                                                                const int* __restrict__ seq_blocks, int batch,
+                                                                int heads, int transposed) {
   const int g = blockIdx.x, h = blockIdx.y;
   const int s = find_seq(seq_blocks, batch, g);
   const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
-  const int64_t tile = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
+  const int64_t base = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
   const int dm = heads * 64;
-  for (int e = threadIdx.x; e < 4096; e += 256) {
-    const int d = e / 64, p = e % 64;
-    v[(int64_t(g) * 64 + slot_token(p)) * dm + h * 64 + d] = vt[tile + e];
+  for (int x = threadIdx.x; x < 4096; x += 256) {
+    const int c = x >> 3, e = x & 7, f = c >> 6, l = c & 63;
+    const int r32 = 32 * (f >> 2) + (l & 31), c8 = 16 * (f & 3) + 8 * (l >> 5) + e;
+    const int token = transposed ? slot_token(c8) : r32;
+    const int d = transposed ? r32 : c8;
+    dst[(int64_t(g) * 64 + token) * dm + h * 64 + d] = packed[base + x];
   }
 }
 
@@ -381,22 +399,23 @@ int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void*
   return check_launch("qkv_bias_split");
 }
 
-int rt_unpack_v_tiles(const void* vt, void* v, const int* seq_blocks_dev, int batch, int total_blocks, int heads,
-                      int dtype, void* stream) {
-  RT_REQUIRE(vt && v && seq_blocks_dev, RT_EINVAL, "NULL pointer");
+int rt_unpack_head_tiles(const void* packed, void* dst, const int* seq_blocks_dev, int batch, int total_blocks,
+                         int heads, int transposed, int dtype, void* stream) {
+  RT_REQUIRE(packed && dst && seq_blocks_dev, RT_EINVAL, "NULL pointer");
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && heads <= 65535, RT_EINVAL,
              "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid(total_blocks, heads);
+  const int tr = transposed ? 1 : 0;
   if (dtype == RT_F16)
-    hipLaunchKernelGGL(unpack_v_tiles_kernel<__half>, grid, dim3(256), 0, st, (const __half*)vt, (__half*)v, seq_blocks_dev, batch, heads);
+    hipLaunchKernelGGL(unpack_head_tiles_kernel<__half>, grid, dim3(256), 0, st, (const __half*)packed, (__half*)dst, seq_blocks_dev, batch, heads, tr);
   else if (dtype == RT_BF16)
-    hipLaunchKernelGGL(unpack_v_tiles_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)vt, (__hip_bfloat16*)v, seq_blocks_dev, batch, heads);
+    hipLaunchKernelGGL(unpack_head_tiles_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)packed, (__hip_bfloat16*)dst, seq_blocks_dev, batch, heads, tr);
   else if (dtype == RT_F32)
-    hipLaunchKernelGGL(unpack_v_tiles_kernel<float>, grid, dim3(256), 0, st, (const float*)vt, (float*)v, seq_blocks_dev, batch, heads);
+    hipLaunchKernelGGL(unpack_head_tiles_kernel<float>, grid, dim3(256), 0, st, (const float*)packed, (float*)dst, seq_blocks_dev, batch, heads, tr);
   else
     return rt::fail(RT_EINVAL, "unknown dtype %d", dtype);
-  return check_launch("unpack_v_tiles");
+  return check_launch("unpack_head_tiles");
 }
 
 }  // extern "C"

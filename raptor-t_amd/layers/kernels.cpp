@@ -5,6 +5,7 @@
 
 #include <cmath>
 #include <mutex>
+#include <vector>
 #include <stdexcept>
 
 namespace sparse_transformers {
@@ -39,24 +40,73 @@ static void require_cuda_contiguous(const torch::Tensor& t, const char* name) {
     throw std::invalid_argument(std::string(name) + " must be a contiguous GPU tensor");
 }
 
-ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* key) {
+namespace {
+struct Deferred {
+  std::mutex m;
+  bool active = false;
+  struct Rec { std::string key; hipEvent_t a, b; };
+  std::vector<Rec> recs;
+};
+Deferred& deferred() { static Deferred d; return d; }
+}  // namespace
+
+void timing_begin() {
+  Deferred& d = deferred();
+  std::lock_guard<std::mutex> lk(d.m);
+  for (auto& r : d.recs) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
+  d.recs.clear();
+  d.active = true;
+}
+
+std::map<std::string, std::pair<double, int64_t>> timing_collect() {
+  Deferred& d = deferred();
+  std::lock_guard<std::mutex> lk(d.m);
+  d.active = false;
+  std::map<std::string, std::pair<double, int64_t>> out;
+  for (auto& r : d.recs) {
+    float ms = 0.f;
+    if (hipEventSynchronize(r.b) == hipSuccess && hipEventElapsedTime(&ms, r.a, r.b) == hipSuccess) {
+      auto& slot = out[r.key];
+      slot.first += double(ms) * 1000.0;
+      slot.second += 1;
+    }
+    (void)hipEventDestroy(r.a);
+    (void)hipEventDestroy(r.b);
+  }
+  d.recs.clear();
+  return out;
+}
+
+ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* key) : key_(key) {
   auto it = info.find(key);
-  if (it == info.end()) return;
-  slot_ = &it->second;
+  if (it != info.end()) slot_ = &it->second;
+  {
+    Deferred& d = deferred();
+    std::lock_guard<std::mutex> lk(d.m);
+    deferred_ = d.active;
+  }
+  if (!slot_ && !deferred_) return;
   hipEvent_t a, b;
-  if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { slot_ = nullptr; return; }
+  if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { slot_ = nullptr; deferred_ = false; return; }
   start_ = a;
   stop_ = b;
   (void)hipEventRecord(a, static_cast<hipStream_t>(current_stream()));
 }
 
 ScopedGpuTimer::~ScopedGpuTimer() {
-  if (!slot_) return;
+  if (!slot_ && !deferred_) return;
   hipEvent_t a = static_cast<hipEvent_t>(start_), b = static_cast<hipEvent_t>(stop_);
   (void)hipEventRecord(b, static_cast<hipStream_t>(current_stream()));
-  (void)hipEventSynchronize(b);
-  float ms = 0.f;
-  if (hipEventElapsedTime(&ms, a, b) == hipSuccess) *slot_ += ms * 1000.0f;
+  if (slot_) {
+    (void)hipEventSynchronize(b);
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, a, b) == hipSuccess) *slot_ += ms * 1000.0f;
+  }
+  if (deferred_) {
+    Deferred& d = deferred();
+    std::lock_guard<std::mutex> lk(d.m);
+    if (d.active) { d.recs.push_back({key_, a, b}); return; }
+  }
   (void)hipEventDestroy(a);
   (void)hipEventDestroy(b);
 }
@@ -70,6 +120,8 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
   require_cuda_contiguous(out, "out");
   if (A.dim() != 2 || B.dim() != 2 || A.size(1) != B.size(0) || out.numel() != A.size(0) * B.size(1))
     throw std::invalid_argument(name + ": shape mismatch");
+  static std::map<std::string, float> no_info;
+  ScopedGpuTimer timer(no_info, "MatMul");
   check(rt_gemm(handle, A.data_ptr(), B.data_ptr(), out.data_ptr(), A.size(0), B.size(1), A.size(1), dtype_code(A),
                 current_stream()), name.c_str());
 }
@@ -80,7 +132,8 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
                                    std::map<std::string, float>& info, bool kernel_fusion) {
   ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel");
   if (head_size != RT_HEAD_DIM) throw std::invalid_argument("head size must be 64");
-  const float scale = 1.0f / std::sqrt(float(head_size));
+  // the attention kernel evaluates the softmax in base 2: fold log2(e) into the Q scale
+  const float scale = 1.4426950408889634f / std::sqrt(float(head_size));
   if (kernel_fusion) {
     check(rt_qkv_bias_split(input_data.data_ptr(), bias.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                             seq_len_info_tensor.data_ptr<int>(), batch_size, block_num, head_num, scale,
@@ -88,25 +141,31 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
     return;
   }
   // Unfused: library ops, one sequence at a time (the reference's own fallback is a
-  // reshape/permute chain, add_bias_and_transpose.cu:219-222).
+  // reshape/permute chain, add_bias_and_transpose.cu:219-222), ending in the fragment order
+  // of the packed layout: [H][n][f>>2][f&3][l>>5][l&31][e] from [H][n][32*(f>>2)+(l&31)][16*(f&3)+8*(l>>5)+e].
   auto sb = seq_len_info_tensor.cpu();
   const int* s = sb.data_ptr<int>();
   const int64_t dm = int64_t(head_num) * head_size;
   auto x = input_data + bias;
-  static const int perm16[16] = {0, 1, 2, 3, 8, 9, 10, 11, 4, 5, 6, 7, 12, 13, 14, 15};
   std::vector<int64_t> slots(64);
-  for (int p = 0; p < 64; ++p) slots[p] = (p & ~15) | perm16[p & 15];
+  for (int p = 0; p < 64; ++p) {
+    const int e = p & 15;
+    slots[p] = (p & ~15) | ((e & 3) | ((e & 4) << 1) | ((e & 8) >> 1));
+  }
   auto slot_idx = torch::tensor(slots, torch::kLong).to(x.device());
   auto qf = q.view({-1}), kf = k.view({-1}), vf = v.view({-1});
+  auto frag = [&](const torch::Tensor& tiles, int64_t n) {       // [H, n, 64(row), 64(col)] -> fragment order
+    return tiles.reshape({head_num, n, 2, 32, 4, 2, 8}).permute({0, 1, 2, 4, 5, 3, 6}).contiguous().view({-1});
+  };
   for (int b = 0; b < batch_size; ++b) {
     const int64_t n = s[b + 1] - s[b], t0 = int64_t(s[b]) * 64, off = t0 * dm;
     auto seq = x.narrow(0, t0, n * 64);
     auto qs = (seq.narrow(1, 0, dm) * scale).view({n, 64, head_num, head_size}).permute({2, 0, 1, 3});
     auto ks = seq.narrow(1, dm, dm).view({n, 64, head_num, head_size}).permute({2, 0, 1, 3});
     auto vs = seq.narrow(1, 2 * dm, dm).view({n, 64, head_num, head_size}).permute({2, 0, 1, 3});
-    qf.narrow(0, off, n * 64 * dm).copy_(qs.contiguous().view({-1}));
-    kf.narrow(0, off, n * 64 * dm).copy_(ks.contiguous().view({-1}));
-    vf.narrow(0, off, n * 64 * dm).copy_(vs.index_select(2, slot_idx).transpose(2, 3).contiguous().view({-1}));
+    qf.narrow(0, off, n * 64 * dm).copy_(frag(qs, n));
+    kf.narrow(0, off, n * 64 * dm).copy_(frag(ks, n));
+    vf.narrow(0, off, n * 64 * dm).copy_(frag(vs.index_select(2, slot_idx).transpose(2, 3), n));
   }
 }
 

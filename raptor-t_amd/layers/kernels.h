@@ -27,7 +27,16 @@ void check(int rc, const char* what);
 // the reference creates a cuBLAS handle per layer object (multi_headed_attention.h:94).
 rt_gemm_ctx* shared_gemm_handle();
 
-// RAII timer: accumulates into info[key] only when the key already exists.
+// Deferred timing: between timing_begin() and timing_collect() every launcher below
+// brackets its kernel with a pair of HIP events on the current stream WITHOUT
+// synchronising; timing_collect() synchronises once and returns, per launcher name,
+// (total microseconds, number of launches).  Lets a harness time kernels inside an
+// otherwise free-running loop.
+void timing_begin();
+std::map<std::string, std::pair<double, int64_t>> timing_collect();
+
+// RAII timer: accumulates into info[key] only when the key already exists (synchronous),
+// and feeds the deferred timing when it is active.
 class ScopedGpuTimer {
  public:
   ScopedGpuTimer(std::map<std::string, float>& info, const char* key);
@@ -35,6 +44,8 @@ class ScopedGpuTimer {
 
  private:
   float* slot_ = nullptr;
+  bool deferred_ = false;
+  const char* key_ = nullptr;
   void* start_ = nullptr;
   void* stop_ = nullptr;
 };

@@ -14,6 +14,10 @@ namespace py = pybind11;
 using namespace sparse_transformers;
 
 PYBIND11_MODULE(raptor_t, m) {
+  m.def("timing_begin", &layers::kernels::timing_begin,
+        "Start bracketing every kernel launcher with HIP events (no synchronisation).");
+  m.def("timing_collect", &layers::kernels::timing_collect,
+        "Synchronise and return {launcher: (total microseconds, launches)} since timing_begin().");
   py::class_<layers::BertAttention>(m, "BertAttention")
       .def(py::init([](torch::Tensor& qkv_weight, torch::Tensor& qkv_bias, torch::Tensor& dense_weight,
                        torch::Tensor& dense_bias, torch::Tensor& layer_norm_weight, torch::Tensor& layer_norm_bias,

@@ -10,6 +10,7 @@ from oracle import attention as oa
 from oracle import layer as ol
 from oracle import metadata as md
 
+LOG2E = 1.4426950408889634
 SLOT_PERM = [0, 1, 2, 3, 8, 9, 10, 11, 4, 5, 6, 7, 12, 13, 14, 15]
 
 
@@ -19,7 +20,9 @@ def slot_tokens():
 
 def pack_heads(x, seq_blocks, transpose_v=False):
     """Token-major [T, H, d] -> the head-major packed layout as a flat tensor (torch statement
-    of the layout documented in include/raptor_t_hip.h)."""
+    of the layout documented in include/raptor_t_hip.h): per (sequence, head, block) a 64x64
+    tile [row][col] (row = token, col = d; for V row = d, col = slot) stored as fragments
+    [row>>5][col>>4][(col>>3)&1][row&31][col&7]."""
     t, heads, d = x.shape
     parts = []
     st = slot_tokens().to(x.device)
@@ -28,6 +31,7 @@ def pack_heads(x, seq_blocks, transpose_v=False):
         blk = x[int(seq_blocks[s]) * 64: int(seq_blocks[s + 1]) * 64].view(n, 64, heads, d).permute(2, 0, 1, 3)
         if transpose_v:
             blk = blk[:, :, st, :].transpose(2, 3)          # [H, n, d, slot]
+        blk = blk.reshape(heads, n, 2, 32, 4, 2, 8).permute(0, 1, 2, 4, 5, 3, 6)
         parts.append(blk.contiguous().view(-1))
     return torch.cat(parts)
 
@@ -44,7 +48,7 @@ def device_plan(capi, seq_lens, heads, seed=0, mode=None, plan_heads=None, devic
 def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0):
     """q, k, v: [T, H, 64] CUDA tensors (q unscaled).  Returns (gpu_out [T, H*64], oracle fp32)."""
     sb, idx, pos, ph, sb_d, idx_d, pos_d = device_plan(capi, seq_lens, heads, seed, mode)
-    qs = (q.float() * 0.125).to(q.dtype)
+    qs = (q.float() * (LOG2E / 8.0)).to(q.dtype)          # the kernel's softmax is base 2
     qp, kp = pack_heads(qs, sb), pack_heads(k, sb)
     vp = pack_heads(v, sb, transpose_v=True)
     out = torch.full((q.shape[0], heads * 64), float("nan"), dtype=q.dtype, device=q.device)
@@ -54,7 +58,7 @@ def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0):
         from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
     capi.bs_attention_fwd(qp, kp, vp, out, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos)
     torch.cuda.synchronize()
-    ref = oa.csr_attention(qs.cpu(), k.cpu(), v.cpu(), sb.tolist(), idx, pos, ph, scale=1.0)
+    ref = oa.csr_attention(qs.cpu(), k.cpu(), v.cpu(), sb.tolist(), idx, pos, ph, scale=1.0 / LOG2E)
     return out, ref
 
 
@@ -77,7 +81,7 @@ def run_layer_case(pkg, seq_lens, hidden, heads, ffn, dtype, seed=0, eps=1e-5, n
         fp, fi = capi.partition_lpt(sb, heads, n_wg)
         from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
     gemm(x, w["qkv_weight"], qkv)
-    capi.qkv_bias_split(qkv, w["qkv_bias"], q, k, vt, sb_d, heads, 1.0 / math.sqrt(hidden // heads))
+    capi.qkv_bias_split(qkv, w["qkv_bias"], q, k, vt, sb_d, heads, LOG2E / math.sqrt(hidden // heads))
     capi.bs_attention_fwd(q, k, vt, ctx, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos)
     gemm(ctx, w["attn_out_weight"], attn)
     capi.bias_residual_layernorm(attn, x, w["attn_out_bias"], w["attn_ln_weight"], w["attn_ln_bias"], eps)
