@@ -96,7 +96,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
         hidden_states.copy_(x0)
         meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
         enc(hidden_states, t, block_limit, spi, spi_t, ppi_t, pp_t, tmp, inter, attn, test_info={},
-            balanced=not args.unbalanced)
+            balanced=args.lpt_plan)
 
     for _ in range(args.warmup):
         step()
@@ -124,7 +124,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": {"workload": name, "layers": layers, "hidden": hidden, "heads": heads, "ffn": ffn,
                    "batch": len(seq_lens), "tokens": t, "seq_lens": seq_lens, "block_limit": block_limit,
-                   "balanced": not args.unbalanced, "async_index": not args.sync_index,
+                   "balanced": args.lpt_plan, "async_index": not args.sync_index,
                    "weights": "random N(0,0.02)", "plan": "per-head HF plan, seed = layer index"},
         "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12,
                      "peak": MFMA_PEAK[dtype] / 1e12, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK[dtype],
@@ -172,10 +172,10 @@ def run_attention_only(args):
     out = torch.empty(t, heads * 64, device="cuda", dtype=torch.float16)
     fp, fi = capi.partition_lpt(sb, heads, args.block_limit)
     fp_d, fi_d = dev(fp), dev(fi)
-    if args.unbalanced:
-        fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads)
-    else:
+    if args.lpt_plan:
         fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads, fi_d, fp_d)
+    else:
+        fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads)
     us = time_kernel(fn, args.steps, args.warmup)
     pairs = block_pairs(sb.tolist(), heads)
     ach = pairs * PAIR_FLOP / (us * 1e-6)
@@ -183,7 +183,7 @@ def run_attention_only(args):
             "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": us / 1e3,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "c2 isolated attention", "block_pairs": pairs, "block_limit": args.block_limit,
-                       "balanced": not args.unbalanced},
+                       "balanced": args.lpt_plan},
             "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12, "peak": 2500.0,
                          "unit": "TFLOP/s", "frac": ach / 2.5e15, "traffic": None}}
 
@@ -216,7 +216,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=["c3", "c2", "c4", "c5", "ref_e2e"])
     ap.add_argument("--block-limit", type=int, default=1024, help="persistent workgroups of the balanced attention launch")
-    ap.add_argument("--unbalanced", action="store_true", help="one workgroup per (head, from-block) unit")
+    ap.add_argument("--lpt-plan", action="store_true",
+                    help="drive attention with the caller's LPT plan (the reference's balanced mode) instead of the kernel's own schedule")
     ap.add_argument("--sync-index", action="store_true", help="build the block index inline instead of on the workers")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=2)

@@ -24,22 +24,19 @@
 //
 // Softmax is evaluated in base 2 (q arrives pre-multiplied by log2(e)/sqrt(d)).  The S^T
 // accumulator starts at minus the row's reference maximum, so the MFMA result feeds exp2
-// directly; the reference is only moved (and O, l rescaled) when a new score exceeds it
-// by more than 2^6, which keeps every P value below 64 and makes the rescale a rare,
-// wave-uniform branch.
+// directly; the reference is only moved (and O, l rescaled) when some P = 2^(score -
+// reference) exceeds 2^6, detected on the packed 16-bit P values: a rare, wave-uniform
+// branch that recomputes the half tile with a proper maximum.
 //
-// Launch without a plan: workgroups enumerate (sequence, head) groups in order, global rows
-// first inside each group, and consecutive workgroup ids are remapped so that each XCD
-// (one L2 per XCD, workgroups are dealt round-robin to the 8 XCDs) walks a contiguous
-// range of groups: the K/V tiles of a (sequence, head) stay in one L2.
-// Launch with an LPT plan: n_wg persistent workgroups walk their unit lists.
+// The kernel is persistent (two workgroups per CU).  Without a plan it makes its own
+// schedule: global rows first, each XCD (one L2 per XCD; workgroups are dealt round-robin to
+// the 8 XCDs) walking its own contiguous share of the (sequence, head) groups, so a group's
+// K/V tiles stay in one L2.  With an LPT plan, n_wg workgroups walk their unit lists.
 //
 // Replaces, from the reference: layers/kernels/sparse_attention.cu:2953-3190 (balanced,
 // persistent workgroups over the LPT plan), :2111-2403 (one workgroup per unit) and the
 // dispatcher :3192-3228.
 #include <hip/hip_runtime.h>
-
-#include <cstdlib>
 
 #include "rt_common.h"
 
@@ -182,13 +179,7 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
 #pragma unroll
           for (int e = 0; e < 16; ++e) sc[t][e] = init;
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-#ifndef RT_X_NOQK
-            sc[t] = Mma<T>::run(kf[t * 4 + c], qf[nt][c], sc[t]);
-#else
-            sc[t][c] += float(kf[t * 4 + c][0]) + float(qf[nt][c][0]);
-#endif
-          }
+          for (int c = 0; c < 4; ++c) sc[t] = Mma<T>::run(kf[t * 4 + c], qf[nt][c], sc[t]);
         }
       };
       // exp2 of the (already shifted) scores -> P as the B operand of the second product:
@@ -201,18 +192,9 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
         for (int s = 0; s < 4; ++s) {
           float p8[8];
 #pragma unroll
-#ifndef RT_X_NOEXP
           for (int e = 0; e < 8; ++e) p8[e] = __builtin_amdgcn_exp2f(sc[s >> 1][8 * (s & 1) + e]);
-#else
-          for (int e = 0; e < 8; ++e) p8[e] = sc[s >> 1][8 * (s & 1) + e];
-#endif
-#ifndef RT_X_NOSUM
           part[s] = Mma<T>::pack(p8, pb[s]);
           top = Mma<T>::max_bits(pb[s], top);
-#else
-          for (int e = 0; e < 8; ++e) pb[s][e] = static_cast<T>(p8[e]);
-          part[s] = 0.f;
-#endif
         }
         psum = (part[0] + part[1]) + (part[2] + part[3]);
         return Mma<T>::over_threshold(top);
@@ -248,29 +230,21 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
         (void)exponentiate();
       }
       // the K fragments are dead once the second query tile's scores are final
-#ifndef RT_X_NOLOAD
       if (nt == 1) {
         __builtin_amdgcn_sched_barrier(0);
         load_tile<T>(kbase + int64_t(bn) * 4096, lane, kf);
         __builtin_amdgcn_sched_barrier(0);
       }
-#endif
       st.l[nt] += psum;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-#ifndef RT_X_NOPV
         for (int s = 0; s < 4; ++s) st.o[t][nt] = Mma<T>::run(vf[t * 4 + s], pb[s], st.o[t][nt]);
-#else
-        for (int s = 0; s < 4; ++s) st.o[t][nt][s] += float(vf[t * 4 + s][0]) + float(pb[s][0]) + float(pb[s][7]);
-#endif
     }
     fresh = false;
-#ifndef RT_X_NOLOAD
     __builtin_amdgcn_sched_barrier(0);
     load_tile<T>(vbase + int64_t(bn) * 4096, lane, vf);
     __builtin_amdgcn_sched_barrier(0);
-#endif
   }
 }
 
@@ -367,9 +341,6 @@ __device__ inline void run_solo(const Args<T>& a, const Unit& u, int lane, T* st
   State st;
   state_init(st);
   stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, lane, qf, st);
-#ifdef RT_X_REPEAT
-  for (int rep = 1; rep < RT_X_REPEAT; ++rep) stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, lane, qf, st);
-#endif
   float w[2];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
@@ -392,9 +363,6 @@ __device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int
   State st;
   state_init(st);
   stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, lane, qf, st);
-#ifdef RT_X_REPEAT
-  for (int rep = 1; rep < RT_X_REPEAT; ++rep) stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, lane, qf, st);
-#endif
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) st.l[nt] += __shfl_xor(st.l[nt], 32, 64);
 
@@ -560,9 +528,6 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
 
 // Two persistent workgroups per CU, a multiple of 8 so that every XCD gets the same number.
 unsigned plan_free_workgroups() {
-#ifdef RT_X_ENVWGS
-  if (const char* e = getenv("RT_X_WGS")) return unsigned(atoi(e));
-#endif
   static unsigned cached = 0;
   if (cached == 0) {
     int dev = 0, cus = 0;
