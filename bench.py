@@ -41,10 +41,18 @@ def block_pairs(seq_blocks, heads):
     return tot * heads
 
 
-def hbm_roofline(name, bytes_per_launch, us_per_launch):
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default workload and scaled by
+# what the same counters read for the QKV split kernel (a copy of known size); the summaries and the commands are
+# in profiles/memory_kernels_c3_traffic.txt.  Only valid for that workload.
+MEASURED_TRAFFIC_C3 = {"bs_attention_kernel": 413.1e6, "bias_residual_layernorm_kernel": 171.4e6,
+                       "bias_gelu_kernel": 457.2e6, "qkv_bias_split_kernel": 342.7e6}
+
+
+def hbm_roofline(name, bytes_per_launch, us_per_launch, traffic=None):
     ach = bytes_per_launch / (us_per_launch * 1e-6)
     return {"kernel": name, "bound": "hbm", "achieved": ach / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": ach / HBM_PEAK, "traffic": None}
+            "frac": ach / HBM_PEAK, "traffic": traffic, "bytes_per_launch": bytes_per_launch,
+            "us_per_launch": us_per_launch}
 
 
 def cpu_baseline_layer(seq_lens, hidden, heads, ffn, layers, sample_seqs, reps=3):
@@ -118,6 +126,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
     att_flops = pairs * PAIR_FLOP
     ach = att_flops / (att_us * 1e-6)
     sz = 2
+    traffic = MEASURED_TRAFFIC_C3 if name.startswith("c3") else {}
     out = {
         "metric": METRIC, "value": len(seq_lens) / (elapsed / args.steps), "unit": "seqs/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step, "ms_per_layer": ms_step / layers,
@@ -128,12 +137,15 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
                    "weights": "random N(0,0.02)", "plan": "per-head HF plan, seed = layer index"},
         "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12,
                      "peak": MFMA_PEAK[dtype] / 1e12, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK[dtype],
-                     "traffic": None, "flop_per_launch": att_flops, "block_pairs": pairs, "us_per_launch": att_us},
+                     "traffic": traffic.get("bs_attention_kernel"), "flop_per_launch": att_flops,
+                     "block_pairs": pairs, "us_per_launch": att_us, "algorithmic_hbm_bytes": 4 * t * hidden * sz},
         "roofline_layernorm": hbm_roofline("bias_residual_layernorm_kernel", 3 * t * hidden * sz,
-                                           per["add_bias_and_layernorm_kernel"]),
-        "roofline_gelu": hbm_roofline("bias_gelu_kernel", 2 * t * ffn * sz, per["add_bias_act_kernel"]),
+                                           per["add_bias_and_layernorm_kernel"],
+                                           traffic.get("bias_residual_layernorm_kernel")),
+        "roofline_gelu": hbm_roofline("bias_gelu_kernel", 2 * t * ffn * sz, per["add_bias_act_kernel"],
+                                      traffic.get("bias_gelu_kernel")),
         "roofline_qkv_split": hbm_roofline("qkv_bias_split_kernel", 2 * t * 3 * hidden * sz,
-                                           per["add_bias_and_transpose_kernel"]),
+                                           per["add_bias_and_transpose_kernel"], traffic.get("qkv_bias_split_kernel")),
         "kernel_us_per_launch": per,
         "kernel_us_per_step": {k: v[0] / args.steps for k, v in timing.items()},
     }

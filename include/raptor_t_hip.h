@@ -154,6 +154,10 @@ int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype
 typedef struct rt_gemm_ctx rt_gemm_ctx;
 int rt_gemm_create(rt_gemm_ctx** ctx);
 int rt_gemm_destroy(rt_gemm_ctx* ctx);
+/* How many hipBLASLt heuristic candidates are timed (once per shape, on the operands of that
+ * shape's first rt_gemm call) before one is kept: 1 = take the library's first suggestion,
+ * default 16. */
+int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates);
 int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c,
             int64_t m, int64_t n, int64_t k, int dtype, void* stream);
 

@@ -21,7 +21,7 @@ EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
-    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm",
+    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
 ]
@@ -60,6 +60,7 @@ def lib():
         L.rt_bias_gelu.argtypes = [vp, vp, L64, I, I, vp]
         L.rt_gemm_create.argtypes = [ctypes.POINTER(vp)]
         L.rt_gemm_destroy.argtypes = [vp]
+        L.rt_gemm_set_tuning.argtypes = [vp, I]
         L.rt_gemm.argtypes = [vp, vp, vp, vp, L64, L64, L64, I, vp]
         L.rt_pipeline_create.argtypes = [ctypes.POINTER(vp), I, I, I, I, I, I, I]
         L.rt_pipeline_publish.argtypes = [vp, i32p, I]
@@ -201,6 +202,9 @@ class Gemm:
     def __init__(self):
         self._h = ctypes.c_void_p()
         check(lib().rt_gemm_create(ctypes.byref(self._h)))
+
+    def set_tuning(self, candidates):
+        check(lib().rt_gemm_set_tuning(self._h, candidates))
 
     def __call__(self, a, b, c):
         m, k = a.shape

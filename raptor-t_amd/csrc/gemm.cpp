@@ -7,6 +7,7 @@
 // failure is reported to the caller instead of ending the process (mat_mul.cpp:60-70).
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <map>
 #include <mutex>
@@ -16,6 +17,7 @@
 
 struct rt_gemm_ctx {
   hipblasLtHandle_t lt = nullptr;
+  int tune_candidates = 16;         // heuristic results timed on a shape's first call (1 = take the first)
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
   int device = 0;
@@ -27,6 +29,9 @@ struct rt_gemm_ctx {
     size_t ws = 0;
   };
   std::map<std::tuple<int64_t, int64_t, int64_t, int>, Plan> plans;
+  // winning solution index per (N, K, dtype): a packed batch changes M with every batch, the
+  // timing run is not repeated for each new M
+  std::map<std::tuple<int64_t, int64_t, int>, int> tuned_index;
 };
 
 namespace {
@@ -37,7 +42,26 @@ namespace {
     if (s_ != HIPBLAS_STATUS_SUCCESS) return rt::fail(RT_EIO, "%s failed with hipblasStatus %d", #expr, int(s_)); \
   } while (0)
 
-int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, rt_gemm_ctx::Plan& p) {
+// Times one candidate on the caller's operands (they are overwritten with the same product).
+float time_algo(rt_gemm_ctx* ctx, const rt_gemm_ctx::Plan& p, const hipblasLtMatmulAlgo_t& algo, const void* a,
+                const void* b, void* c, hipStream_t st, hipEvent_t e0, hipEvent_t e1) {
+  const float alpha = 1.0f, beta = 0.0f;
+  const int reps = 3;
+  for (int r = 0; r <= reps; ++r) {               // the first run is a warm-up
+    if (r == 1 && hipEventRecord(e0, st) != hipSuccess) return -1.f;
+    if (hipblasLtMatmul(ctx->lt, p.desc, &alpha, b, p.la, a, p.lb, &beta, c, p.lc, c, p.lc, &algo, ctx->workspace,
+                        ctx->workspace_bytes, st) != HIPBLAS_STATUS_SUCCESS)
+      return -1.f;
+  }
+  float ms = -1.f;
+  if (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+      hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
+    return -1.f;
+  return ms / reps;
+}
+
+int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, rt_gemm_ctx::Plan& p, const void* a,
+              const void* b, void* c, hipStream_t st) {
   const hipDataType t = dtype == RT_F16 ? HIP_R_16F : (dtype == RT_BF16 ? HIP_R_16BF : HIP_R_32F);
   LT_TRY(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   hipblasOperation_t nop = HIPBLAS_OP_N;
@@ -51,15 +75,45 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, rt_g
   LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
   LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ctx->workspace_bytes,
                                                sizeof(ctx->workspace_bytes)));
-  hipblasLtMatmulHeuristicResult_t res[4];
+  constexpr int MAX_CAND = 64;
+  hipblasLtMatmulHeuristicResult_t res[MAX_CAND];
   int found = 0;
-  hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(ctx->lt, p.desc, p.la, p.lb, p.lc, p.lc, pref, 4, res, &found);
+  const int want = ctx->tune_candidates < 1 ? 1 : (ctx->tune_candidates > MAX_CAND ? MAX_CAND : ctx->tune_candidates);
+  hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(ctx->lt, p.desc, p.la, p.lb, p.lc, p.lc, pref, want, res, &found);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (hs != HIPBLAS_STATUS_SUCCESS || found == 0)
     return rt::fail(RT_ENOSYS, "hipBLASLt has no algorithm for M=%lld N=%lld K=%lld dtype=%d (status %d)", (long long)m,
                     (long long)n, (long long)k, dtype, int(hs));
-  p.algo = res[0].algo;
-  p.ws = res[0].workspaceSize;
+  int best = -1;
+  auto tuned = ctx->tuned_index.find(std::make_tuple(n, k, dtype));
+  if (tuned != ctx->tuned_index.end())
+    for (int i = 0; i < found && best < 0; ++i)
+      if (res[i].state == HIPBLAS_STATUS_SUCCESS && hipblaslt_ext::getIndexFromAlgo(res[i].algo) == tuned->second) best = i;
+  if (best >= 0) {
+    p.algo = res[best].algo;
+    p.ws = res[best].workspaceSize;
+    return RT_OK;
+  }
+  best = 0;
+  // The library's first suggestion is often not the fastest for these tall, K=768 shapes: time the
+  // candidates once per shape on the caller's own operands (skipped while a graph is being captured).
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (found > 1 && hipStreamIsCapturing(st, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone) {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+      float best_ms = -1.f;
+      for (int i = 0; i < found; ++i) {
+        if (res[i].state != HIPBLAS_STATUS_SUCCESS || res[i].workspaceSize > ctx->workspace_bytes) continue;
+        const float ms = time_algo(ctx, p, res[i].algo, a, b, c, st, e0, e1);
+        if (ms > 0.f && (best_ms < 0.f || ms < best_ms)) { best_ms = ms; best = i; }
+      }
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+  }
+  p.algo = res[best].algo;
+  p.ws = res[best].workspaceSize;
+  ctx->tuned_index[std::make_tuple(n, k, dtype)] = hipblaslt_ext::getIndexFromAlgo(res[best].algo);
   return RT_OK;
 }
 
@@ -100,6 +154,14 @@ int rt_gemm_destroy(rt_gemm_ctx* ctx) {
   return RT_OK;
 }
 
+int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates) {
+  RT_REQUIRE(ctx, RT_EINVAL, "NULL context");
+  RT_REQUIRE(candidates >= 1 && candidates <= 64, RT_EINVAL, "candidates=%d out of range [1, 64]", candidates);
+  std::lock_guard<std::mutex> lk(ctx->m);
+  ctx->tune_candidates = candidates;
+  return RT_OK;
+}
+
 int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int dtype,
             void* stream) {
   RT_REQUIRE(ctx && a && b && c, RT_EINVAL, "NULL argument");
@@ -113,7 +175,7 @@ int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c, int64_t m, 
     auto it = ctx->plans.find(key);
     if (it == ctx->plans.end()) {
       rt_gemm_ctx::Plan p;
-      int rc = make_plan(ctx, m, n, k, dtype, p);
+      int rc = make_plan(ctx, m, n, k, dtype, p, a, b, c, static_cast<hipStream_t>(stream));
       if (rc) { free_plan(p); return rc; }
       it = ctx->plans.emplace(key, p).first;
     }
