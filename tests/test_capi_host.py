@@ -178,3 +178,17 @@ def test_pipeline_ordering_and_termination(capi):
     pipe2.close()
     pipe.close()            # terminate with idle workers: must join, not hang
     pipe.close()            # idempotent
+
+
+def test_pipeline_is_race_free_under_thread_sanitizer():
+    """Builds the host pipeline with -fsanitize=thread and runs the stress driver
+    (tests/host/pipeline_stress.cpp): publish / acquire / release orders, double signals,
+    destruction right after a publish.  Any data race makes the run fail."""
+    import subprocess
+    csrc = os.path.join(graft.ROOT, "raptor-t_amd", "csrc")
+    subprocess.check_call(["make", "-C", csrc, "tsan_test"], stdout=subprocess.DEVNULL, stderr=subprocess.STDOUT)
+    exe = os.path.join(graft.ROOT, "raptor-t_amd", "build", "pipeline_stress_tsan")
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 exitcode=66")
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-4000:]
+    assert "pipeline_stress OK" in res.stdout and "ThreadSanitizer" not in res.stderr
