@@ -144,27 +144,27 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
                                     const int* __restrict__ row, int first, int step, int cnt, int n, int lane,
                                     const typename Mma<T>::v8 (&qf)[2][4], State& st) {
   typedef typename Mma<T>::v8 v8;
-  if (first >= cnt) return;
-  int chunk = first >> 6;
-  int ids = (chunk * 64 + lane < cnt) ? row[chunk * 64 + lane] : 0;
-  auto block_of = [&](int j) {                        // j is wave-uniform
-    if ((j >> 6) != chunk) {
-      chunk = j >> 6;
-      ids = (chunk * 64 + lane < cnt) ? row[chunk * 64 + lane] : 0;
-    }
-    const int b = __builtin_amdgcn_readlane(ids, j & 63);
+  v8 kf[8], vf[8];
+  bool fresh = true;                                  // no reference maximum yet
+  // Rows longer than 64 entries are walked in chunks of 64: the ids are only (re)loaded between
+  // chunks, so inside the tile loop the only outstanding memory operations are the tile
+  // prefetches and the waits on them can be exact.
+  for (int j = first; j < cnt;) {
+  const int chunk = j >> 6;
+  const int hi = min(cnt, (chunk + 1) * 64);
+  const int ids = (chunk * 64 + lane < cnt) ? row[chunk * 64 + lane] : 0;
+  auto block_of = [&](int e) {                        // e is wave-uniform and inside the chunk
+    const int b = __builtin_amdgcn_readlane(ids, e & 63);
     return b < 0 ? 0 : (b >= n ? n - 1 : b);
   };
-  v8 kf[8], vf[8];
   {
-    const int b = block_of(first);
+    const int b = block_of(j);
     load_tile<T>(kbase + int64_t(b) * 4096, lane, kf);
     load_tile<T>(vbase + int64_t(b) * 4096, lane, vf);
   }
-  bool fresh = true;                                  // no reference maximum yet
-  for (int j = first; j < cnt; j += step) {
+  for (; j < hi; j += step) {
     const int jn = j + step;
-    const bool more = jn < cnt;
+    const bool more = jn < hi;
     // the last iteration re-requests its own tile: loads stay unconditional, so they keep
     // their place in the instruction stream (a branch would sink them next to their use)
     const int bn = block_of(more ? jn : j);
@@ -245,6 +245,7 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
     __builtin_amdgcn_sched_barrier(0);
     load_tile<T>(vbase + int64_t(bn) * 4096, lane, vf);
     __builtin_amdgcn_sched_barrier(0);
+  }
   }
 }
 
