@@ -161,6 +161,15 @@ int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates);
 int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c,
             int64_t m, int64_t n, int64_t k, int dtype, void* stream);
 
+/* The same product with the epilogue fused into the GEMM: C = A . B + bias[N]
+ * (RT_EPILOGUE_BIAS) or C = gelu_tanh(A . B + bias[N]) (RT_EPILOGUE_BIAS_GELU).  The second
+ * replaces the pair kernels::MatMul + kernels::add_bias_act_kernel of BertIntermediate
+ * (layers/bert_intermediate.cpp:22-30) with one pass over the [M, N] output; bias has the
+ * dtype of the operands. */
+enum { RT_EPILOGUE_NONE = 0, RT_EPILOGUE_BIAS = 1, RT_EPILOGUE_BIAS_GELU = 2 };
+int rt_gemm_bias_act(rt_gemm_ctx* ctx, const void* a, const void* b, const void* bias, void* c,
+                     int64_t m, int64_t n, int64_t k, int epilogue, int dtype, void* stream);
+
 /* ------------------------------------------------------- metadata / stream pipeline */
 
 /* Replaces Semaphore + MetaData + the per-layer std::async index workers

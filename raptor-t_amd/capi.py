@@ -16,12 +16,14 @@ RT_F16, RT_BF16, RT_F32 = 0, 1, 2
 RT_PLAN_HF, RT_PLAN_REFERENCE, RT_PLAN_EXPLICIT = 0, 1, 2
 RT_POLICY_REFERENCE_PATCHED, RT_POLICY_HF_UPSTREAM = 0, 1
 RT_EINVAL, RT_ENOMEM, RT_EIO, RT_ENOSYS, RT_ECANCELED = -22, -12, -5, -38, -125
+RT_EPILOGUE_NONE, RT_EPILOGUE_BIAS, RT_EPILOGUE_BIAS_GELU = 0, 1, 2
 
 EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm",
+    "rt_gemm_bias_act",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
 ]
@@ -62,6 +64,7 @@ def lib():
         L.rt_gemm_destroy.argtypes = [vp]
         L.rt_gemm_set_tuning.argtypes = [vp, I]
         L.rt_gemm.argtypes = [vp, vp, vp, vp, L64, L64, L64, I, vp]
+        L.rt_gemm_bias_act.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
         L.rt_pipeline_create.argtypes = [ctypes.POINTER(vp), I, I, I, I, I, I, I]
         L.rt_pipeline_publish.argtypes = [vp, i32p, I]
         L.rt_pipeline_acquire.argtypes = [vp, I, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), i32p,
@@ -210,6 +213,14 @@ class Gemm:
         m, k = a.shape
         n = b.shape[1]
         check(lib().rt_gemm(self._h, _dp(a), _dp(b), _dp(c), m, n, k, _dtype_code(a), _stream()))
+        return c
+
+    def bias_act(self, a, b, bias, c, epilogue=RT_EPILOGUE_BIAS_GELU):
+        """c = a @ b + bias, through the tanh GELU when epilogue is RT_EPILOGUE_BIAS_GELU, in one kernel."""
+        m, k = a.shape
+        n = b.shape[1]
+        check(lib().rt_gemm_bias_act(self._h, _dp(a), _dp(b), _dp(bias), _dp(c), m, n, k, epilogue, _dtype_code(a),
+                                     _stream()))
         return c
 
     def close(self):

@@ -5,6 +5,11 @@
 // with the operands swapped to express a row-major product in a column-major library and
 // accumulates in fp16; the same operand swap is used here, the accumulator is fp32, and a
 // failure is reported to the caller instead of ending the process (mat_mul.cpp:60-70).
+//
+// rt_gemm_bias_act runs the same product with the bias add, and optionally the tanh GELU, in
+// the GEMM's epilogue: what BertIntermediate does with MatMul followed by add_bias_act_kernel
+// (layers/bert_intermediate.cpp:22-30, layers/kernels/add_bias_act.cu:114-133) in one pass over
+// the output.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 #include <hipblaslt/hipblaslt-ext.hpp>
@@ -28,10 +33,11 @@ struct rt_gemm_ctx {
     hipblasLtMatmulAlgo_t algo;
     size_t ws = 0;
   };
-  std::map<std::tuple<int64_t, int64_t, int64_t, int>, Plan> plans;
-  // winning solution index per (N, K, dtype): a packed batch changes M with every batch, the
-  // timing run is not repeated for each new M
-  std::map<std::tuple<int64_t, int64_t, int>, int> tuned_index;
+  // keyed by (M, N, K, dtype, epilogue)
+  std::map<std::tuple<int64_t, int64_t, int64_t, int, int>, Plan> plans;
+  // winning solution index per (N, K, dtype, epilogue): a packed batch changes M with every
+  // batch, the timing run is not repeated for each new M
+  std::map<std::tuple<int64_t, int64_t, int, int>, int> tuned_index;
 };
 
 namespace {
@@ -60,13 +66,21 @@ float time_algo(rt_gemm_ctx* ctx, const rt_gemm_ctx::Plan& p, const hipblasLtMat
   return ms / reps;
 }
 
-int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, rt_gemm_ctx::Plan& p, const void* a,
-              const void* b, void* c, hipStream_t st) {
+// epilogue: RT_EPILOGUE_NONE, or bias / bias + GELU along the N columns of the row-major output
+// (the rows of the column-major problem handed to the library, where it expects the bias).
+int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int epilogue, const void* bias,
+              rt_gemm_ctx::Plan& p, const void* a, const void* b, void* c, hipStream_t st) {
   const hipDataType t = dtype == RT_F16 ? HIP_R_16F : (dtype == RT_BF16 ? HIP_R_16BF : HIP_R_32F);
   LT_TRY(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   hipblasOperation_t nop = HIPBLAS_OP_N;
   LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &nop, sizeof(nop)));
   LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &nop, sizeof(nop)));
+  if (epilogue != RT_EPILOGUE_NONE) {
+    hipblasLtEpilogue_t ep = epilogue == RT_EPILOGUE_BIAS_GELU ? HIPBLASLT_EPILOGUE_GELU_BIAS : HIPBLASLT_EPILOGUE_BIAS;
+    LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &ep, sizeof(ep)));
+    LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
+    LT_TRY(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &t, sizeof(t)));
+  }
   // column-major view: C^T[N,M] = B^T[N,K] . A^T[K,M]
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.la, t, n, k, n));
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.lb, t, k, m, k));
@@ -85,7 +99,7 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, rt_g
     return rt::fail(RT_ENOSYS, "hipBLASLt has no algorithm for M=%lld N=%lld K=%lld dtype=%d (status %d)", (long long)m,
                     (long long)n, (long long)k, dtype, int(hs));
   int best = -1;
-  auto tuned = ctx->tuned_index.find(std::make_tuple(n, k, dtype));
+  auto tuned = ctx->tuned_index.find(std::make_tuple(n, k, dtype, epilogue));
   if (tuned != ctx->tuned_index.end())
     for (int i = 0; i < found && best < 0; ++i)
       if (res[i].state == HIPBLAS_STATUS_SUCCESS && hipblaslt_ext::getIndexFromAlgo(res[i].algo) == tuned->second) best = i;
@@ -113,7 +127,7 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, rt_g
   }
   p.algo = res[best].algo;
   p.ws = res[best].workspaceSize;
-  ctx->tuned_index[std::make_tuple(n, k, dtype)] = hipblaslt_ext::getIndexFromAlgo(res[best].algo);
+  ctx->tuned_index[std::make_tuple(n, k, dtype, epilogue)] = hipblaslt_ext::getIndexFromAlgo(res[best].algo);
   return RT_OK;
 }
 
@@ -162,29 +176,49 @@ int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates) {
   return RT_OK;
 }
 
-int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int dtype,
-            void* stream) {
+}  // extern "C"
+
+namespace {
+
+int run_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, const void* bias, void* c, int64_t m, int64_t n, int64_t k,
+             int epilogue, int dtype, void* stream) {
   RT_REQUIRE(ctx && a && b && c, RT_EINVAL, "NULL argument");
   RT_REQUIRE(m >= 0 && n > 0 && k > 0, RT_EINVAL, "bad shape M=%lld N=%lld K=%lld", (long long)m, (long long)n, (long long)k);
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
   if (m == 0) return RT_OK;
-  rt_gemm_ctx::Plan* plan;
-  {
-    std::lock_guard<std::mutex> lk(ctx->m);
-    auto key = std::make_tuple(m, n, k, dtype);
-    auto it = ctx->plans.find(key);
-    if (it == ctx->plans.end()) {
-      rt_gemm_ctx::Plan p;
-      int rc = make_plan(ctx, m, n, k, dtype, p, a, b, c, static_cast<hipStream_t>(stream));
-      if (rc) { free_plan(p); return rc; }
-      it = ctx->plans.emplace(key, p).first;
-    }
-    plan = &it->second;
-  }
   const float alpha = 1.0f, beta = 0.0f;
+  // the plan's descriptor carries the bias pointer: set and used under the lock
+  std::lock_guard<std::mutex> lk(ctx->m);
+  auto key = std::make_tuple(m, n, k, dtype, epilogue);
+  auto it = ctx->plans.find(key);
+  if (it == ctx->plans.end()) {
+    rt_gemm_ctx::Plan p;
+    int rc = make_plan(ctx, m, n, k, dtype, epilogue, bias, p, a, b, c, static_cast<hipStream_t>(stream));
+    if (rc) { free_plan(p); return rc; }
+    it = ctx->plans.emplace(key, p).first;
+  }
+  rt_gemm_ctx::Plan* plan = &it->second;
+  if (epilogue != RT_EPILOGUE_NONE)
+    LT_TRY(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
   LT_TRY(hipblasLtMatmul(ctx->lt, plan->desc, &alpha, b, plan->la, a, plan->lb, &beta, c, plan->lc, c, plan->lc,
                          &plan->algo, ctx->workspace, ctx->workspace_bytes, static_cast<hipStream_t>(stream)));
   return RT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int dtype,
+            void* stream) {
+  return run_gemm(ctx, a, b, nullptr, c, m, n, k, RT_EPILOGUE_NONE, dtype, stream);
+}
+
+int rt_gemm_bias_act(rt_gemm_ctx* ctx, const void* a, const void* b, const void* bias, void* c, int64_t m, int64_t n,
+                     int64_t k, int epilogue, int dtype, void* stream) {
+  RT_REQUIRE(epilogue == RT_EPILOGUE_BIAS || epilogue == RT_EPILOGUE_BIAS_GELU, RT_EINVAL, "unknown epilogue %d", epilogue);
+  RT_REQUIRE(bias, RT_EINVAL, "NULL bias");
+  return run_gemm(ctx, a, b, bias, c, m, n, k, epilogue, dtype, stream);
 }
 
 }  // extern "C"

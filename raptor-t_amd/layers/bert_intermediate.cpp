@@ -14,6 +14,10 @@ BertIntermediate::BertIntermediate(torch::Tensor dense_weight, torch::Tensor den
 
 std::map<std::string, float> BertIntermediate::operator()(const torch::Tensor& input_tensor, torch::Tensor& output_tensor,
                                                           std::map<std::string, float>& info, bool kernel_fusion) const {
+  if (kernel_fusion && kernels::gemm_epilogue_fusion()) {
+    kernels::MatMulBiasGelu(input_tensor, dense_weight_, dense_bias_, output_tensor, handle_, info, "BertIntermediate");
+    return info;
+  }
   kernels::MatMul(input_tensor, false, dense_weight_, false, 1.0, output_tensor, 0.0, handle_, "BertIntermediate");
   kernels::add_bias_act_kernel(dense_bias_, output_tensor, int(input_tensor.size(0)), int(dense_bias_.size(0)), info,
                                kernel_fusion);

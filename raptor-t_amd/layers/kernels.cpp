@@ -3,6 +3,7 @@
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <cmath>
 #include <mutex>
 #include <vector>
@@ -124,6 +125,26 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
   ScopedGpuTimer timer(no_info, "MatMul");
   check(rt_gemm(handle, A.data_ptr(), B.data_ptr(), out.data_ptr(), A.size(0), B.size(1), A.size(1), dtype_code(A),
                 current_stream()), name.c_str());
+}
+
+namespace {
+std::atomic<bool> g_epilogue_fusion{true};
+}
+void set_gemm_epilogue_fusion(bool on) { g_epilogue_fusion.store(on); }
+bool gemm_epilogue_fusion() { return g_epilogue_fusion.load(); }
+
+void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch::Tensor& bias, torch::Tensor& out,
+                    rt_gemm_ctx* handle, std::map<std::string, float>& info, const std::string& name) {
+  require_cuda_contiguous(A, "A");
+  require_cuda_contiguous(B, "B");
+  require_cuda_contiguous(bias, "bias");
+  require_cuda_contiguous(out, "out");
+  if (A.dim() != 2 || B.dim() != 2 || A.size(1) != B.size(0) || out.numel() != A.size(0) * B.size(1) ||
+      bias.numel() != B.size(1) || bias.scalar_type() != A.scalar_type())
+    throw std::invalid_argument(name + ": shape or dtype mismatch");
+  ScopedGpuTimer timer(info, "MatMul_bias_gelu");
+  check(rt_gemm_bias_act(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), B.size(1),
+                         A.size(1), RT_EPILOGUE_BIAS_GELU, dtype_code(A), current_stream()), name.c_str());
 }
 
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,

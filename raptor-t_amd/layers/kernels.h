@@ -55,6 +55,16 @@ class ScopedGpuTimer {
 void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b_trans, float alpha,
             torch::Tensor& out, float beta, rt_gemm_ctx* handle, const std::string& name);
 
+// MatMul followed by add_bias_act_kernel, as one GEMM with the bias add and the tanh GELU in
+// its epilogue (what BertIntermediate's pair of calls, layers/bert_intermediate.cpp:22-30,
+// computes).  Times itself under "MatMul_bias_gelu".
+void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch::Tensor& bias, torch::Tensor& out,
+                    rt_gemm_ctx* handle, std::map<std::string, float>& info, const std::string& name);
+// Whether BertIntermediate uses MatMulBiasGelu when kernel_fusion is asked for (default) or
+// keeps the GEMM and the bias + GELU kernel apart.
+void set_gemm_epilogue_fusion(bool on);
+bool gemm_epilogue_fusion();
+
 // layers/kernels/add_bias_and_transpose.cu:212-233
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,
                                    torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,

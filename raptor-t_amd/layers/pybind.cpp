@@ -16,6 +16,10 @@ using namespace sparse_transformers;
 PYBIND11_MODULE(raptor_t, m) {
   m.def("timing_begin", &layers::kernels::timing_begin,
         "Start bracketing every kernel launcher with HIP events (no synchronisation).");
+  m.def("set_gemm_epilogue_fusion", &layers::kernels::set_gemm_epilogue_fusion,
+        "BertIntermediate with kernel_fusion runs bias + GELU in the GEMM's epilogue (True, the default) or as the "
+        "separate add_bias_act kernel (False).");
+  m.def("gemm_epilogue_fusion", &layers::kernels::gemm_epilogue_fusion);
   m.def("timing_collect", &layers::kernels::timing_collect,
         "Synchronise and return {launcher: (total microseconds, launches)} since timing_begin().");
   py::class_<layers::BertAttention>(m, "BertAttention")

@@ -181,6 +181,36 @@ def test_gemm_matches_torch(capi, dtype):
     gemm.close()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gemm_bias_gelu_epilogue_matches_oracle(capi, dtype):
+    """The fused epilogue against the oracle's bias + tanh GELU applied to an fp32 product, and against
+    the library's own two-kernel path (GEMM, then bias_gelu)."""
+    say("gemm epilogue", dtype)
+    g = torch.Generator().manual_seed(1)
+    gemm = capi.Gemm()
+    for m, n, k in [(832, 3072, 768), (64, 1024, 256), (1, 768, 768)]:
+        a = torch.randn(m, k, generator=g).to(dtype).cuda()
+        b = (torch.randn(k, n, generator=g) * 0.05).to(dtype).cuda()
+        bias = torch.randn(n, generator=g).to(dtype).cuda()
+        fused = torch.empty(m, n, dtype=dtype, device="cuda")
+        gemm.bias_act(a, b, bias, fused)
+        plain = torch.empty(m, n, dtype=dtype, device="cuda")
+        gemm.bias_act(a, b, bias, plain, capi.RT_EPILOGUE_BIAS)
+        two = torch.empty(m, n, dtype=dtype, device="cuda")
+        gemm(a, b, two)
+        capi.bias_gelu(two, bias)
+        torch.cuda.synchronize()
+        prod = a.double().cpu() @ b.double().cpu()
+        want = ol.bias_gelu(prod, bias.cpu())
+        tol = 2e-2 if dtype == torch.float16 else 6e-2         # the two-kernel path rounds the product to T first
+        assert (fused.float().cpu() - want).abs().max().item() <= tol
+        assert (two.float().cpu() - want).abs().max().item() <= tol
+        assert (plain.double().cpu() - (prod + bias.double().cpu())).abs().max().item() <= tol
+    with pytest.raises(capi.RaptorError):
+        gemm.bias_act(a, b, bias, fused, epilogue=7)
+    gemm.close()
+
+
 @pytest.mark.parametrize("dtype,hidden,heads,ffn,n_wg", [
     (torch.float16, 768, 12, 3072, 0), (torch.bfloat16, 1024, 16, 4096, 64), (torch.float16, 768, 12, 3072, 160)])
 def test_encoder_layer_matches_oracle(capi, dtype, hidden, heads, ffn, n_wg):

@@ -94,15 +94,22 @@ def test_fused_and_unfused_paths_agree(mb, ut):
     x = torch.randn(t, hidden, generator=g).to(dtype).cuda()
     spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, 64, heads)
     outs = []
-    for fused in (True, False):
+    # bias + GELU in the GEMM's epilogue / as its own kernel / as torch operators
+    for fused, epilogue in ((True, True), (True, False), (False, False)):
+        mb.cxx.set_gemm_epilogue_fusion(epilogue)
         meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
         h = x.clone()
         new = lambda wd: torch.empty(t, wd, dtype=dtype, device="cuda")
+        mb.cxx.timing_begin()
         out, _ = layer(h, spi, spi_t, ppi_t, pp_t, new(ffn), new(hidden), new(hidden), 64, kernel_fusion=fused)
-        torch.cuda.synchronize()
+        ran = mb.cxx.timing_collect()
+        assert ("MatMul_bias_gelu" in ran) == (fused and epilogue)
+        assert ("add_bias_act_kernel" in ran) == (not (fused and epilogue))
         outs.append(out.float().cpu())
+    mb.cxx.set_gemm_epilogue_fusion(True)
     meta.terminate_thread()
     assert (outs[0] - outs[1]).abs().max().item() <= 2e-2
+    assert (outs[0] - outs[2]).abs().max().item() <= 2e-2
 
 
 def test_api_rejects_mismatched_batch(mb, ut):
