@@ -146,6 +146,17 @@ int rt_bias_residual_layernorm(void* out, const void* residual, const void* bias
  * out = gelu_tanh(out + bias), in place on out[rows, width]; width a multiple of 8. */
 int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype, void* stream);
 
+/* Replaces the PyTorch operators of BertEmbeddings.__call__ (python/modeling_bert.py:47-63):
+ * out[t] = LayerNorm(word[input_ids[t]] + position[position_ids[t]] + token_type[token_type_ids[t]])
+ * * gamma + beta for the T tokens of a packed batch, written in out_dtype (the reference casts to
+ * fp16).  Tables [vocab | max_pos | type_vocab, hidden], gamma and beta have table_dtype (fp32 in the
+ * reference); ids are int32 device arrays and are clamped into their table; hidden a multiple of 8. */
+int rt_embed_layernorm(const int* input_ids, const int* position_ids, const int* token_type_ids,
+                       const void* word, const void* position, const void* token_type,
+                       const void* gamma, const void* beta, void* out, int64_t rows, int hidden,
+                       int vocab, int max_pos, int type_vocab, float eps, int table_dtype,
+                       int out_dtype, void* stream);
+
 /* ---------------------------------------------------------------------- dense GEMM */
 
 /* Replaces kernels::MatMul (layers/kernels/mat_mul.cpp:9-96): row-major

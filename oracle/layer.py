@@ -8,6 +8,7 @@ Test infrastructure (see oracle/__init__.py).  Follows
     layers/bert_output.cpp:7-44                        call order and buffer roles
   * python/modeling_big_bird.py:1318-1329, :1424-1451, :1564-1567  the same glue in the
     reference's oracle (SelfOutput, Intermediate, Output, feed_forward_chunk)
+  * python/modeling_bert.py:47-63                      embedding sum + LayerNorm(eps 1e-12)
 Weights are stored `[in, out]` as the reference stores them
 (python/modeling_bert.py:84-91, :107-113, :137-163); the fused QKV weight is Q|K|V.
 """
@@ -25,6 +26,18 @@ GELU_C1 = 0.044715
 def bias_residual_layernorm(x, residual, bias, gamma, beta, eps):
     h = x.float() + bias.float() + residual.float()
     return F.layer_norm(h, (h.shape[-1],), gamma.float(), beta.float(), eps)
+
+
+def embeddings_layernorm(input_ids, position_ids, token_type_ids, word, position, token_type, gamma, beta,
+                         eps=1e-12):
+    """Packed-input front end of the reference (python/modeling_bert.py:53-62): rows of the three tables
+    are gathered and summed in the order word + token_type + position, then LayerNorm.  Written out with
+    explicit indexing and moments (not nn.Embedding / F.layer_norm, which the tests pin it against)."""
+    x = (word.double()[input_ids.long()] + token_type.double()[token_type_ids.long()]
+         + position.double()[position_ids.long()])
+    mean = x.mean(dim=-1, keepdim=True)
+    var = ((x - mean) ** 2).mean(dim=-1, keepdim=True)            # biased, as LayerNorm defines it
+    return ((x - mean) / torch.sqrt(var + eps) * gamma.double() + beta.double()).float()
 
 
 def bias_gelu(x, bias):

@@ -22,7 +22,7 @@ EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
-    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm",
+    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm",
     "rt_gemm_bias_act",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
@@ -64,6 +64,7 @@ def lib():
         L.rt_gemm_destroy.argtypes = [vp]
         L.rt_gemm_set_tuning.argtypes = [vp, I]
         L.rt_gemm.argtypes = [vp, vp, vp, vp, L64, L64, L64, I, vp]
+        L.rt_embed_layernorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, L64, I, I, I, I, ctypes.c_float, I, I, vp]
         L.rt_gemm_bias_act.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
         L.rt_pipeline_create.argtypes = [ctypes.POINTER(vp), I, I, I, I, I, I, I]
         L.rt_pipeline_publish.argtypes = [vp, i32p, I]
@@ -197,6 +198,24 @@ def bias_residual_layernorm(out, residual, bias, gamma, beta, eps):
 def bias_gelu(out, bias):
     rows, width = out.shape
     check(lib().rt_bias_gelu(_dp(out), _dp(bias), rows, width, _dtype_code(out), _stream()))
+
+
+def embed_layernorm(input_ids, position_ids, token_type_ids, word, position, token_type, gamma, beta, out, eps=1e-12):
+    """out[t] = LN(word[ids[t]] + position[pos[t]] + token_type[type[t]]) * gamma + beta; ids are int32 device
+    tensors, the tables / gamma / beta share one dtype, out has the encoder's."""
+    import torch
+    for t in (input_ids, position_ids, token_type_ids):
+        if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous() or t.numel() != out.shape[0]:
+            raise ValueError("ids must be contiguous int32 device tensors with one entry per output row")
+    for t in (position, token_type, gamma, beta):
+        if t.dtype != word.dtype:
+            raise ValueError("tables, gamma and beta must share one dtype")
+    rows, hidden = out.shape
+    check(lib().rt_embed_layernorm(_dp(input_ids), _dp(position_ids), _dp(token_type_ids), _dp(word), _dp(position),
+                                   _dp(token_type), _dp(gamma), _dp(beta), _dp(out), rows, hidden, word.shape[0],
+                                   position.shape[0], token_type.shape[0], eps, _dtype_code(word), _dtype_code(out),
+                                   _stream()))
+    return out
 
 
 class Gemm:

@@ -1,15 +1,19 @@
 // Memory-bound kernels of the encoder layer for gfx950 (wave64): fused
-// bias+residual+LayerNorm, bias+GELU(tanh form), and the QKV bias/scale/head split that
-// writes the head-major packed layout the attention kernel reads.
+// bias+residual+LayerNorm, bias+GELU(tanh form), the QKV bias/scale/head split that
+// writes the head-major packed layout the attention kernel reads, and the embedding
+// gather + LayerNorm that produces the encoder's packed input.
 //
-// All three move 16 bytes per lane per access so that every wave issues full 1 KiB
+// All of them move 16 bytes per lane per access so that every wave issues full 1 KiB
 // requests; statistics and the activation are computed in fp32.
 //
 // Replaces, from the reference: layers/kernels/add_bias_and_layernorm.cu:191-285,
-// layers/kernels/add_bias_act.cu:41-48,86-133, layers/kernels/add_bias_and_transpose.cu:118-233.
+// layers/kernels/add_bias_act.cu:41-48,86-133, layers/kernels/add_bias_and_transpose.cu:118-233,
+// and the PyTorch operators of BertEmbeddings.__call__ (python/modeling_bert.py:47-63).
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "rt_common.h"
 
@@ -189,11 +193,166 @@ int ln_dispatch(void* out, const void* res, const void* bias, const void* gamma,
   return RT_OK;
 }
 
+// ---- embedding gather + LayerNorm ---------------------------------------------------------
+// out[t] = LN(word[ids[t]] + position[pos_ids[t]] + type[type_ids[t]]) * gamma + beta, written in
+// the encoder's dtype.  Tables, gamma and beta are of type TT (fp32 as the reference keeps them,
+// or a 16-bit type).  Ids outside a table are clamped into it.
+template <typename TT> __device__ inline void load8(const TT* p, float* f) {
+  constexpr int N = Vec<TT>::N;
+#pragma unroll
+  for (int i = 0; i < 8; i += N) Vec<TT>::load(p + i, f + i);
+}
+template <typename TO> __device__ inline void store8_out(TO* p, const float* f) {
+  constexpr int N = Vec<TO>::N;
+#pragma unroll
+  for (int i = 0; i < 8; i += N) Vec<TO>::store(p + i, f + i);
+}
+__device__ inline int clamp_id(int v, int n) { return v < 0 ? 0 : (v >= n ? n - 1 : v); }
+
+template <typename TT, typename TO> struct EmbedArgs {
+  const int* ids; const int* pos_ids; const int* type_ids;
+  const TT* word; const TT* pos; const TT* type; const TT* gamma; const TT* beta;
+  TO* out;
+  int64_t rows;
+  int vocab, max_pos, type_vocab;
+  float eps;
+};
+
+// One row per group of G lanes; each lane keeps CHUNKS runs of 8 elements: hidden = CHUNKS * G * 8.
+template <typename TT, typename TO, int CHUNKS, int G>
+__global__ __launch_bounds__(256) void embed_layernorm_kernel(EmbedArgs<TT, TO> a) {
+  constexpr int HIDDEN = CHUNKS * G * 8;
+  const int lane = threadIdx.x % G;
+  const int64_t row = int64_t(blockIdx.x) * (256 / G) + threadIdx.x / G;
+  if (row >= a.rows) return;
+  const TT* w = a.word + int64_t(clamp_id(a.ids[row], a.vocab)) * HIDDEN;
+  const TT* p = a.pos + int64_t(clamp_id(a.pos_ids[row], a.max_pos)) * HIDDEN;
+  const TT* t = a.type + int64_t(clamp_id(a.type_ids[row], a.type_vocab)) * HIDDEN;
+  float x[CHUNKS][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int col = (c * G + lane) * 8;
+    float u[8], v[8], z[8];
+    load8<TT>(w + col, u);
+    load8<TT>(p + col, v);
+    load8<TT>(t + col, z);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { x[c][i] = u[i] + z[i] + v[i]; sum += x[c][i]; }
+  }
+  const float mean = group_sum<G>(sum) * (1.0f / HIDDEN);
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { const float d = x[c][i] - mean; sq += d * d; }
+  const float rstd = rsqrtf(group_sum<G>(sq) * (1.0f / HIDDEN) + a.eps);
+  TO* o = a.out + row * HIDDEN;
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int col = (c * G + lane) * 8;
+    float g[8], b[8], y[8];
+    load8<TT>(a.gamma + col, g);
+    load8<TT>(a.beta + col, b);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (x[c][i] - mean) * rstd * g[i] + b[i];
+    store8_out<TO>(o + col, y);
+  }
+}
+
+// Any hidden that is a multiple of 8: one wave per row, three sweeps over the table rows.
+template <typename TT, typename TO>
+__global__ __launch_bounds__(256) void embed_layernorm_generic_kernel(EmbedArgs<TT, TO> a, int hidden) {
+  const int lane = threadIdx.x % 64;
+  const int64_t row = int64_t(blockIdx.x) * 4 + threadIdx.x / 64;
+  if (row >= a.rows) return;
+  const TT* w = a.word + int64_t(clamp_id(a.ids[row], a.vocab)) * hidden;
+  const TT* p = a.pos + int64_t(clamp_id(a.pos_ids[row], a.max_pos)) * hidden;
+  const TT* t = a.type + int64_t(clamp_id(a.type_ids[row], a.type_vocab)) * hidden;
+  auto value = [&](int col, float* x) {
+    float u[8], v[8], z[8];
+    load8<TT>(w + col, u); load8<TT>(p + col, v); load8<TT>(t + col, z);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = u[i] + z[i] + v[i];
+  };
+  float sum = 0.f;
+  for (int col = lane * 8; col < hidden; col += 512) {
+    float x[8];
+    value(col, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += x[i];
+  }
+  const float mean = group_sum<64>(sum) / hidden;
+  float sq = 0.f;
+  for (int col = lane * 8; col < hidden; col += 512) {
+    float x[8];
+    value(col, x);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { const float d = x[i] - mean; sq += d * d; }
+  }
+  const float rstd = rsqrtf(group_sum<64>(sq) / hidden + a.eps);
+  TO* o = a.out + row * hidden;
+  for (int col = lane * 8; col < hidden; col += 512) {
+    float x[8], g[8], b[8], y[8];
+    value(col, x);
+    load8<TT>(a.gamma + col, g);
+    load8<TT>(a.beta + col, b);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (x[i] - mean) * rstd * g[i] + b[i];
+    store8_out<TO>(o + col, y);
+  }
+}
+
+template <typename TT, typename TO, int CHUNKS, int G>
+void launch_embed(const EmbedArgs<TT, TO>& a, hipStream_t st) {
+  const int rows_per_wg = 256 / G;
+  const unsigned grid = unsigned((a.rows + rows_per_wg - 1) / rows_per_wg);
+  hipLaunchKernelGGL((embed_layernorm_kernel<TT, TO, CHUNKS, G>), dim3(grid), dim3(256), 0, st, a);
+}
+
+template <typename TT, typename TO>
+void embed_dispatch(const EmbedArgs<TT, TO>& a, int hidden, hipStream_t st) {
+  if (hidden % 256 == 0) {
+    switch (hidden / 256) {          // chunks per lane with 32 lanes per row
+      case 1: launch_embed<TT, TO, 1, 32>(a, st); return;
+      case 2: launch_embed<TT, TO, 2, 32>(a, st); return;
+      case 3: launch_embed<TT, TO, 3, 32>(a, st); return;      // 768
+      case 4: launch_embed<TT, TO, 4, 32>(a, st); return;      // 1024
+      case 6: launch_embed<TT, TO, 3, 64>(a, st); return;
+      case 8: launch_embed<TT, TO, 4, 64>(a, st); return;
+      default: break;
+    }
+  }
+  const unsigned grid = unsigned((a.rows + 3) / 4);
+  hipLaunchKernelGGL((embed_layernorm_generic_kernel<TT, TO>), dim3(grid), dim3(256), 0, st, a, hidden);
+}
+
+template <typename TT>
+int embed_out_dispatch(const int* ids, const int* pos_ids, const int* type_ids, const void* word, const void* pos,
+                       const void* type, const void* gamma, const void* beta, void* out, int64_t rows, int hidden,
+                       int vocab, int max_pos, int type_vocab, float eps, int out_dtype, hipStream_t st) {
+  auto run = [&](auto* o) {
+    typedef typename std::remove_pointer<decltype(o)>::type TO;
+    EmbedArgs<TT, TO> a{ids, pos_ids, type_ids, static_cast<const TT*>(word), static_cast<const TT*>(pos),
+                        static_cast<const TT*>(type), static_cast<const TT*>(gamma), static_cast<const TT*>(beta),
+                        o, rows, vocab, max_pos, type_vocab, eps};
+    embed_dispatch<TT, TO>(a, hidden, st);
+  };
+  if (out_dtype == RT_F16) run(static_cast<__half*>(out));
+  else if (out_dtype == RT_BF16) run(static_cast<__hip_bfloat16*>(out));
+  else run(static_cast<float*>(out));
+  return RT_OK;
+}
+
 // ---- bias + GELU (tanh form) ------------------------------------------------------------
-// gelu(x) = 0.5 x (1 + tanh(u)), u = c0 (x + c1 x^3)  ==  x / (1 + exp(-2u)).
+// gelu(x) = 0.5 x (1 + tanh(u)), u = c0 (x + c1 x^3)  ==  x / (1 + exp(-2u))
+//         = x / (1 + 2^(x (k0 + k1 x^2))),  k0 = -2 c0 log2(e), k1 = k0 c1:
+// three multiplies and one fma around the two transcendental instructions.
 __device__ inline float gelu_tanh(float x) {
-  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  return x * __frcp_rn(1.0f + __expf(-2.0f * u));
+  constexpr float K0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  constexpr float K1 = K0 * 0.044715f;
+  const float t = x * fmaf(K1, x * x, K0);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
 }
 
 // The launch makes the grid stride a multiple of the row width, so a thread always lands
@@ -416,6 +575,38 @@ int rt_unpack_head_tiles(const void* packed, void* dst, const int* seq_blocks_de
   else
     return rt::fail(RT_EINVAL, "unknown dtype %d", dtype);
   return check_launch("unpack_head_tiles");
+}
+
+int rt_embed_layernorm(const int* input_ids, const int* position_ids, const int* token_type_ids, const void* word,
+                       const void* position, const void* token_type, const void* gamma, const void* beta, void* out,
+                       int64_t rows, int hidden, int vocab, int max_pos, int type_vocab, float eps, int table_dtype,
+                       int out_dtype, void* stream) {
+  RT_REQUIRE(rows >= 0 && rows < (int64_t(1) << 31), RT_EINVAL, "rows=%lld out of range", (long long)rows);
+  RT_REQUIRE(word && position && token_type && gamma && beta, RT_EINVAL, "NULL table pointer");
+  RT_REQUIRE(rows == 0 || (input_ids && position_ids && token_type_ids && out), RT_EINVAL, "NULL id or output pointer");
+  RT_REQUIRE(hidden > 0 && hidden % 8 == 0, RT_EINVAL, "hidden=%d must be a positive multiple of 8", hidden);
+  RT_REQUIRE(vocab > 0 && max_pos > 0 && type_vocab > 0, RT_EINVAL, "empty table: vocab=%d max_pos=%d type_vocab=%d", vocab,
+             max_pos, type_vocab);
+  RT_REQUIRE(table_dtype == RT_F16 || table_dtype == RT_BF16 || table_dtype == RT_F32, RT_EINVAL, "unknown table dtype %d",
+             table_dtype);
+  RT_REQUIRE(out_dtype == RT_F16 || out_dtype == RT_BF16 || out_dtype == RT_F32, RT_EINVAL, "unknown output dtype %d",
+             out_dtype);
+  RT_REQUIRE(aligned16(word) && aligned16(position) && aligned16(token_type) && aligned16(gamma) && aligned16(beta) &&
+                 aligned16(out), RT_EINVAL, "tables, gamma, beta and out must be 16-byte aligned");
+  if (rows == 0) return RT_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (table_dtype == RT_F32)
+    embed_out_dispatch<float>(input_ids, position_ids, token_type_ids, word, position, token_type, gamma, beta, out, rows,
+                              hidden, vocab, max_pos, type_vocab, eps, out_dtype, st);
+  else if (table_dtype == RT_F16)
+    embed_out_dispatch<__half>(input_ids, position_ids, token_type_ids, word, position, token_type, gamma, beta, out, rows,
+                               hidden, vocab, max_pos, type_vocab, eps, out_dtype, st);
+  else
+    embed_out_dispatch<__hip_bfloat16>(input_ids, position_ids, token_type_ids, word, position, token_type, gamma, beta,
+                                       out, rows, hidden, vocab, max_pos, type_vocab, eps, out_dtype, st);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return rt::fail(RT_EIO, "embed_layernorm launch failed: %s", hipGetErrorString(e));
+  return RT_OK;
 }
 
 }  // extern "C"

@@ -6,6 +6,7 @@
 #include <atomic>
 #include <cmath>
 #include <mutex>
+#include <set>
 #include <vector>
 #include <stdexcept>
 
@@ -47,13 +48,15 @@ struct Deferred {
   bool active = false;
   struct Rec { std::string key; hipEvent_t a, b; };
   std::vector<Rec> recs;
+  std::set<std::string> only;          // empty: every launcher is timed
 };
 Deferred& deferred() { static Deferred d; return d; }
 }  // namespace
 
-void timing_begin() {
+void timing_begin(const std::vector<std::string>& only) {
   Deferred& d = deferred();
   std::lock_guard<std::mutex> lk(d.m);
+  d.only = std::set<std::string>(only.begin(), only.end());
   for (auto& r : d.recs) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
   d.recs.clear();
   d.active = true;
@@ -84,7 +87,7 @@ ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* k
   {
     Deferred& d = deferred();
     std::lock_guard<std::mutex> lk(d.m);
-    deferred_ = d.active;
+    deferred_ = d.active && (d.only.empty() || d.only.count(key) != 0);
   }
   if (!slot_ && !deferred_) return;
   hipEvent_t a, b;

@@ -11,6 +11,7 @@
 
 #include <map>
 #include <string>
+#include <vector>
 
 #include "../../include/raptor_t_hip.h"
 
@@ -32,7 +33,7 @@ rt_gemm_ctx* shared_gemm_handle();
 // synchronising; timing_collect() synchronises once and returns, per launcher name,
 // (total microseconds, number of launches).  Lets a harness time kernels inside an
 // otherwise free-running loop.
-void timing_begin();
+void timing_begin(const std::vector<std::string>& only = {});
 std::map<std::string, std::pair<double, int64_t>> timing_collect();
 
 // RAII timer: accumulates into info[key] only when the key already exists (synchronous),

@@ -14,8 +14,9 @@ namespace py = pybind11;
 using namespace sparse_transformers;
 
 PYBIND11_MODULE(raptor_t, m) {
-  m.def("timing_begin", &layers::kernels::timing_begin,
-        "Start bracketing every kernel launcher with HIP events (no synchronisation).");
+  m.def("timing_begin", &layers::kernels::timing_begin, py::arg("only") = std::vector<std::string>(),
+        "Start bracketing kernel launchers with HIP events (no synchronisation): every launcher, or only the "
+        "named ones (each pair of events costs a few microseconds between kernels).");
   m.def("set_gemm_epilogue_fusion", &layers::kernels::set_gemm_epilogue_fusion,
         "BertIntermediate with kernel_fusion runs bias + GELU in the GEMM's epilogue (True, the default) or as the "
         "separate add_bias_act kernel (False).");

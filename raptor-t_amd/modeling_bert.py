@@ -24,6 +24,8 @@ try:
 except ImportError as e:            # no silent fallback: the layer API is the product
     raise ImportError("the raptor_t extension is not built: run __graft_entry__.build() (%s)" % e)
 
+from . import capi
+
 roctx = torch.cuda.nvtx             # torch maps these ranges onto roctx on ROCm
 
 
@@ -38,31 +40,34 @@ def create_empty_if_none(tensor, shape, device, dtype=torch.float16):
 
 
 class BertEmbeddings:
-    """Word + position + token-type embeddings and LayerNorm(eps 1e-12), kept in PyTorch as in
-    the reference (:27-69); returns the packed [T, D] activations in the encoder's dtype."""
+    """Word + position + token-type embeddings and LayerNorm(eps 1e-12) of the packed input
+    (reference: python/modeling_bert.py:27-69, there PyTorch operators): one gather + LayerNorm
+    kernel writing the packed [T, D] activations in the encoder's dtype.  The tables stay in fp32
+    as the reference keeps them."""
 
     def __init__(self, word_embeddings_weight, position_embeddings_weight, token_type_embeddings_weight,
                  layerNorm_weight, layerNorm_bias, pad_token_id: int = 0, dtype=torch.float16, device="cuda"):
-        self.word_embeddings = nn.Embedding.from_pretrained(word_embeddings_weight.detach().float(), freeze=True,
-                                                            padding_idx=pad_token_id).to(device)
-        self.position_embeddings = nn.Embedding.from_pretrained(position_embeddings_weight.detach().float(),
-                                                                freeze=True).to(device)
-        self.token_type_embeddings = nn.Embedding.from_pretrained(token_type_embeddings_weight.detach().float(),
-                                                                  freeze=True).to(device)
-        hidden = word_embeddings_weight.shape[1]
-        self.LayerNorm = nn.LayerNorm(hidden, eps=1e-12).to(device)
-        with torch.no_grad():
-            self.LayerNorm.weight.copy_(layerNorm_weight)
-            self.LayerNorm.bias.copy_(layerNorm_bias)
+        prep = lambda w: w.detach().to(device=device, dtype=torch.float32).contiguous()
+        self.word_embeddings = prep(word_embeddings_weight)
+        self.position_embeddings = prep(position_embeddings_weight)
+        self.token_type_embeddings = prep(token_type_embeddings_weight)
+        self.gamma = prep(layerNorm_weight)
+        self.beta = prep(layerNorm_bias)
+        self.pad_token_id = pad_token_id          # kept for the reference's signature; a lookup needs no padding row
         self.dtype = dtype
+        self.eps = 1e-12
 
     @torch.no_grad()
     def __call__(self, input_ids=None, position_ids=None, token_type_ids=None, output=None):
         if input_ids is None or position_ids is None or token_type_ids is None:
             raise ValueError("input_ids, position_ids and token_type_ids are all required")
-        emb = (self.word_embeddings(input_ids.long()) + self.token_type_embeddings(token_type_ids.long())
-               + self.position_embeddings(position_ids.long()))
-        return self.LayerNorm(emb).to(self.dtype).contiguous()
+        dev = self.word_embeddings.device
+        ids = [t.to(device=dev, dtype=torch.int32).contiguous().view(-1) for t in (input_ids, position_ids, token_type_ids)]
+        if output is None:
+            output = torch.empty(ids[0].numel(), self.word_embeddings.shape[1], dtype=self.dtype, device=dev)
+        capi.embed_layernorm(ids[0], ids[1], ids[2], self.word_embeddings, self.position_embeddings,
+                             self.token_type_embeddings, self.gamma, self.beta, output, self.eps)
+        return output
 
     @staticmethod
     def from_torch(bert_embedding, dtype=torch.float16):

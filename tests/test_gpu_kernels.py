@@ -181,6 +181,34 @@ def test_gemm_matches_torch(capi, dtype):
     gemm.close()
 
 
+@pytest.mark.parametrize("table_dtype,out_dtype,hidden", [
+    (torch.float32, torch.float16, 768), (torch.float32, torch.bfloat16, 1024), (torch.float16, torch.float16, 768),
+    (torch.float32, torch.float32, 1536), (torch.float32, torch.float16, 200)])
+def test_embed_layernorm_matches_oracle(capi, table_dtype, out_dtype, hidden):
+    say("embed", table_dtype, out_dtype, hidden)
+    g = torch.Generator().manual_seed(3)
+    vocab, max_pos, types, t = 1000, 4096, 2, 1000 + 37
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(table_dtype)
+    word, pos, typ, gamma, beta = mk(vocab, hidden), mk(max_pos, hidden), mk(types, hidden), mk(hidden), mk(hidden)
+    ids = torch.randint(0, vocab, (t,), generator=g, dtype=torch.int32)
+    pids = torch.randint(0, max_pos, (t,), generator=g, dtype=torch.int32)
+    tids = torch.randint(0, types, (t,), generator=g, dtype=torch.int32)
+    ids[0], ids[1], pids[2] = -5, vocab + 9, max_pos          # outside their tables: clamped to the nearest row
+    out = torch.empty(t, hidden, dtype=out_dtype, device="cuda")
+    capi.embed_layernorm(ids.cuda(), pids.cuda(), tids.cuda(), word.cuda(), pos.cuda(), typ.cuda(), gamma.cuda(),
+                         beta.cuda(), out)
+    torch.cuda.synchronize()
+    want = ol.embeddings_layernorm(ids.clamp(0, vocab - 1), pids.clamp(0, max_pos - 1), tids, word, pos, typ, gamma, beta)
+    tol = {torch.float16: 2e-2, torch.bfloat16: 6e-2, torch.float32: 1e-4}[out_dtype]
+    assert (out.float().cpu() - want).abs().max().item() <= tol
+    empty = torch.empty(0, hidden, dtype=out_dtype, device="cuda")
+    z = torch.empty(0, dtype=torch.int32, device="cuda")
+    capi.embed_layernorm(z, z, z, word.cuda(), pos.cuda(), typ.cuda(), gamma.cuda(), beta.cuda(), empty)
+    with pytest.raises(capi.RaptorError):
+        capi.embed_layernorm(ids.cuda(), pids.cuda(), tids.cuda(), word.cuda()[:, :-4].contiguous(), pos.cuda(), typ.cuda(),
+                             gamma.cuda(), beta.cuda(), torch.empty(t, hidden - 4, dtype=out_dtype, device="cuda"))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_gemm_bias_gelu_epilogue_matches_oracle(capi, dtype):
     """The fused epilogue against the oracle's bias + tanh GELU applied to an fp32 product, and against

@@ -52,3 +52,29 @@ def test_layer_composition_matches_plain_torch_modules():
     i = F.gelu(a @ w["inter_weight"] + w["inter_bias"], approximate="tanh")
     want = F.layer_norm(i @ w["out_weight"] + w["out_bias"] + a, (hid,), w["out_ln_weight"], w["out_ln_bias"], 1e-5)
     assert (got - want).abs().max().item() < 2e-5
+
+
+def test_embeddings_layernorm_matches_torch_modules_and_hand_case():
+    """The restatement indexes and normalises by hand; torch's own Embedding + LayerNorm modules (what the
+    reference calls, python/modeling_bert.py:31-36,53-62) are the independent answer.  A dropped table,
+    a swapped id stream or an unbiased variance each fail it."""
+    g = torch.Generator().manual_seed(5)
+    vocab, max_pos, types, hidden, t = 97, 33, 2, 24, 50
+    word, pos, typ = (torch.randn(n, hidden, generator=g) for n in (vocab, max_pos, types))
+    gamma, beta = torch.randn(hidden, generator=g), torch.randn(hidden, generator=g)
+    ids = torch.randint(0, vocab, (t,), generator=g)
+    pids = torch.randint(0, max_pos, (t,), generator=g)
+    tids = torch.randint(0, types, (t,), generator=g)
+    got = ol.embeddings_layernorm(ids, pids, tids, word, pos, typ, gamma, beta, eps=1e-12)
+    ln = torch.nn.LayerNorm(hidden, eps=1e-12)
+    with torch.no_grad():
+        ln.weight.copy_(gamma)
+        ln.bias.copy_(beta)
+        want = ln(torch.nn.functional.embedding(ids, word) + torch.nn.functional.embedding(tids, typ)
+                  + torch.nn.functional.embedding(pids, pos))
+    assert (got - want).abs().max().item() <= 2e-5
+    # hand case: rows sum to [1, 3] -> mean 2, biased variance 1 -> [-1, 1] * gamma + beta
+    w = torch.tensor([[0.0, 1.0], [5.0, 5.0]]); p = torch.tensor([[1.0, 1.0]]); ty = torch.tensor([[0.0, 1.0]])
+    out = ol.embeddings_layernorm(torch.tensor([0]), torch.tensor([0]), torch.tensor([0]), w, p, ty,
+                                  torch.tensor([2.0, 3.0]), torch.tensor([0.5, -0.5]), eps=0.0)
+    assert torch.allclose(out, torch.tensor([[-1.5, 2.5]]), atol=1e-6)
