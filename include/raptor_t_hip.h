@@ -165,9 +165,11 @@ int rt_embed_layernorm(const int* input_ids, const int* position_ids, const int*
 typedef struct rt_gemm_ctx rt_gemm_ctx;
 int rt_gemm_create(rt_gemm_ctx** ctx);
 int rt_gemm_destroy(rt_gemm_ctx* ctx);
-/* How many hipBLASLt heuristic candidates are timed (once per shape, on the operands of that
- * shape's first rt_gemm call) before one is kept: 1 = take the library's first suggestion,
- * default 16. */
+/* How many hipBLASLt heuristic candidates are timed (once per (N, K, dtype, epilogue), on the
+ * operands of the first rt_gemm call of that kind) before one is kept: 1 = take the library's
+ * first suggestion, default 16; RT_GEMM_TUNE_ALL = every solution of the library that accepts
+ * the problem (seconds per kind, once per process). */
+#define RT_GEMM_TUNE_ALL (-1)
 int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates);
 int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c,
             int64_t m, int64_t n, int64_t k, int dtype, void* stream);

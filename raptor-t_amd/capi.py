@@ -17,6 +17,7 @@ RT_PLAN_HF, RT_PLAN_REFERENCE, RT_PLAN_EXPLICIT = 0, 1, 2
 RT_POLICY_REFERENCE_PATCHED, RT_POLICY_HF_UPSTREAM = 0, 1
 RT_EINVAL, RT_ENOMEM, RT_EIO, RT_ENOSYS, RT_ECANCELED = -22, -12, -5, -38, -125
 RT_EPILOGUE_NONE, RT_EPILOGUE_BIAS, RT_EPILOGUE_BIAS_GELU = 0, 1, 2
+RT_GEMM_TUNE_ALL = -1
 
 EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",

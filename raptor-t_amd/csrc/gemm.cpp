@@ -15,6 +15,7 @@
 #include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <map>
+#include <vector>
 #include <mutex>
 #include <tuple>
 
@@ -90,19 +91,53 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int 
   LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ctx->workspace_bytes,
                                                sizeof(ctx->workspace_bytes)));
   constexpr int MAX_CAND = 64;
-  hipblasLtMatmulHeuristicResult_t res[MAX_CAND];
+  std::vector<hipblasLtMatmulHeuristicResult_t> res(MAX_CAND);
   int found = 0;
   const int want = ctx->tune_candidates < 1 ? 1 : (ctx->tune_candidates > MAX_CAND ? MAX_CAND : ctx->tune_candidates);
-  hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(ctx->lt, p.desc, p.la, p.lb, p.lc, p.lc, pref, want, res, &found);
+  hipblasStatus_t hs =
+      hipblasLtMatmulAlgoGetHeuristic(ctx->lt, p.desc, p.la, p.lb, p.lc, p.lc, pref, want, res.data(), &found);
   hipblasLtMatmulPreferenceDestroy(pref);
   if (hs != HIPBLAS_STATUS_SUCCESS || found == 0)
     return rt::fail(RT_ENOSYS, "hipBLASLt has no algorithm for M=%lld N=%lld K=%lld dtype=%d (status %d)", (long long)m,
                     (long long)n, (long long)k, dtype, int(hs));
+  res.resize(found);
+  if (ctx->tune_candidates == RT_GEMM_TUNE_ALL && !ctx->tuned_index.count(std::make_tuple(n, k, dtype, epilogue))) {
+    // every solution the library has for these types, filtered to the ones that accept this problem
+    std::vector<hipblasLtMatmulHeuristicResult_t> all;
+    if (hipblaslt_ext::getAllAlgos(ctx->lt, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, HIPBLAS_OP_N, HIPBLAS_OP_N, t, t, t, t,
+                                   HIPBLAS_COMPUTE_32F, all) == HIPBLAS_STATUS_SUCCESS) {
+      const float one = 1.0f, zero = 0.0f;
+      for (auto& r : all) {
+        size_t ws = 0;
+        if (hipblaslt_ext::matmulIsAlgoSupported(ctx->lt, p.desc, &one, p.la, p.lb, &zero, p.lc, p.lc, r.algo, ws) !=
+                HIPBLAS_STATUS_SUCCESS || ws > ctx->workspace_bytes)
+          continue;
+        r.workspaceSize = ws;
+        r.state = HIPBLAS_STATUS_SUCCESS;
+        res.push_back(r);
+      }
+      found = int(res.size());
+    }
+  }
   int best = -1;
   auto tuned = ctx->tuned_index.find(std::make_tuple(n, k, dtype, epilogue));
   if (tuned != ctx->tuned_index.end())
     for (int i = 0; i < found && best < 0; ++i)
       if (res[i].state == HIPBLAS_STATUS_SUCCESS && hipblaslt_ext::getIndexFromAlgo(res[i].algo) == tuned->second) best = i;
+  if (best < 0 && tuned != ctx->tuned_index.end()) {
+    // the winner of an exhaustive search need not be among the heuristic's suggestions for this M
+    std::vector<int> index{tuned->second};
+    std::vector<hipblasLtMatmulHeuristicResult_t> byindex;
+    const float one = 1.0f, zero = 0.0f;
+    size_t ws = 0;
+    if (hipblaslt_ext::getAlgosFromIndex(ctx->lt, index, byindex) == HIPBLAS_STATUS_SUCCESS && !byindex.empty() &&
+        hipblaslt_ext::matmulIsAlgoSupported(ctx->lt, p.desc, &one, p.la, p.lb, &zero, p.lc, p.lc, byindex[0].algo, ws) ==
+            HIPBLAS_STATUS_SUCCESS && ws <= ctx->workspace_bytes) {
+      p.algo = byindex[0].algo;
+      p.ws = ws;
+      return RT_OK;
+    }
+  }
   if (best >= 0) {
     p.algo = res[best].algo;
     p.ws = res[best].workspaceSize;
@@ -170,7 +205,8 @@ int rt_gemm_destroy(rt_gemm_ctx* ctx) {
 
 int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates) {
   RT_REQUIRE(ctx, RT_EINVAL, "NULL context");
-  RT_REQUIRE(candidates >= 1 && candidates <= 64, RT_EINVAL, "candidates=%d out of range [1, 64]", candidates);
+  RT_REQUIRE((candidates >= 1 && candidates <= 64) || candidates == RT_GEMM_TUNE_ALL, RT_EINVAL,
+             "candidates=%d must be in [1, 64] or RT_GEMM_TUNE_ALL", candidates);
   std::lock_guard<std::mutex> lk(ctx->m);
   ctx->tune_candidates = candidates;
   return RT_OK;

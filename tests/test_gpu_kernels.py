@@ -181,6 +181,29 @@ def test_gemm_matches_torch(capi, dtype):
     gemm.close()
 
 
+def test_gemm_exhaustive_tuning_keeps_results(capi):
+    """RT_GEMM_TUNE_ALL times every library solution once per (N, K, dtype); later calls with another M reuse
+    the winner by index.  Results must not depend on the tuning mode."""
+    say("gemm tune all")
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(320, 256, generator=g).half().cuda()
+    b = (torch.randn(256, 512, generator=g) * 0.05).half().cuda()
+    want = a.float().cpu() @ b.float().cpu()
+    for mode in (1, capi.RT_GEMM_TUNE_ALL):
+        gemm = capi.Gemm()
+        gemm.set_tuning(mode)
+        for rows in (320, 192):                       # the second M takes the cached winner
+            c = torch.empty(rows, 512, dtype=torch.float16, device="cuda")
+            gemm(a[:rows].contiguous(), b, c)
+            torch.cuda.synchronize()
+            assert (c.float().cpu() - want[:rows]).abs().max().item() <= 2e-2
+        gemm.close()
+    gemm = capi.Gemm()
+    with pytest.raises(capi.RaptorError):
+        gemm.set_tuning(0)
+    gemm.close()
+
+
 @pytest.mark.parametrize("table_dtype,out_dtype,hidden", [
     (torch.float32, torch.float16, 768), (torch.float32, torch.bfloat16, 1024), (torch.float16, torch.float16, 768),
     (torch.float32, torch.float32, 1536), (torch.float32, torch.float16, 200)])
