@@ -24,7 +24,7 @@ try:
 except ImportError as e:            # no silent fallback: the layer API is the product
     raise ImportError("the raptor_t extension is not built: run __graft_entry__.build() (%s)" % e)
 
-from . import capi
+from . import capi, checkpoint
 
 roctx = torch.cuda.nvtx             # torch maps these ranges onto roctx on ROCm
 
@@ -242,6 +242,29 @@ class BertModelNoPooler:
         eps = model.config.layer_norm_eps if eps is None else eps
         return BertModelNoPooler(BertEmbeddings.from_torch(model.embeddings, dtype),
                                  BertEncoder.from_torch(model.encoder, async_, dtype, eps))
+
+
+def _model_from_checkpoint(path, heads=None, async_=True, dtype=torch.float16, eps=None, device="cuda"):
+    emb, layers, cfg = checkpoint.load(path)
+    heads = cfg.get("num_attention_heads") if heads is None else heads
+    if heads is None:
+        raise ValueError("no config.json beside the checkpoint: pass heads=")
+    eps = cfg.get("layer_norm_eps", 1e-12) if eps is None else eps
+    act = cfg.get("hidden_act", "gelu_new")
+    if act not in ("gelu_new", "gelu_pytorch_tanh", "gelu_fast"):
+        raise ValueError("the layer applies the tanh GELU; this checkpoint's hidden_act is %r" % act)
+    embeddings = BertEmbeddings(emb["word_embeddings.weight"], emb["position_embeddings.weight"],
+                                emb["token_type_embeddings.weight"], emb["LayerNorm.weight"], emb["LayerNorm.bias"],
+                                pad_token_id=cfg.get("pad_token_id", 0), dtype=dtype, device=device)
+    dev = lambda w: {k: v.detach().to(device=device, dtype=dtype).contiguous() for k, v in w.items()}
+    return BertModelNoPooler(embeddings, BertEncoder.from_weights([dev(w) for w in layers], heads, async_, eps))
+
+
+BertModelNoPooler.from_local_checkpoint = staticmethod(_model_from_checkpoint)
+BertModelNoPooler.from_local_checkpoint.__doc__ = (
+    "Builds the model from a HuggingFace BigBird / BERT checkpoint on disk (a directory with config.json and "
+    "model.safetensors or pytorch_model.bin, or the weight file itself): the on-disk counterpart of from_torch "
+    "(reference python/modeling_bert.py:62-69, :137-163).  Nothing is fetched over the network.")
 
 
 def random_layer_weights(hidden, ffn, generator, std=0.02, dtype=torch.float16, device="cuda"):

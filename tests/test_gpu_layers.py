@@ -2,6 +2,7 @@
 callers) against the CPU oracle and against the HuggingFace BigBird model installed on the
 box, on the same seeded inputs and the same random-block plan."""
 import importlib
+import json
 
 import numpy as np
 import pytest
@@ -160,3 +161,41 @@ def test_from_torch_matches_huggingface_bigbird(mb, ut, length):
     err = (out.float().cpu() - want).abs().max().item()
     say("  hf err", err)
     assert err <= 2e-2
+
+
+def test_local_checkpoint_matches_huggingface_bigbird(mb, ut, tmp_path):
+    """A HuggingFace BigBird checkpoint written to disk (safetensors + config.json), read back by
+    from_local_checkpoint, against the HuggingFace model that wrote it."""
+    say("local checkpoint")
+    from safetensors.torch import save_file
+    from transformers import BigBirdConfig, BigBirdModel
+    torch.manual_seed(1)
+    length = 896
+    cfg = BigBirdConfig(vocab_size=500, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        intermediate_size=256, max_position_embeddings=4096, attention_type="block_sparse",
+                        block_size=64, num_random_blocks=3, hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+    hf = BigBirdModel(cfg, add_pooling_layer=False).cuda().train()
+    save_file({k: v.detach().cpu().contiguous() for k, v in hf.state_dict().items()}, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(cfg.to_json_string())
+    ids = torch.randint(1, 500, (1, length), device="cuda")
+    with torch.no_grad():
+        want = hf(input_ids=ids).last_hidden_state[0].float().cpu()
+    model = mb.BertModelNoPooler.from_local_checkpoint(str(tmp_path))
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo([length], 64, 48, 2)
+    meta.update_meta_data(length, spi[-1] + 1, total_comp, spi)
+    pos = torch.arange(length, device="cuda")
+    inter = torch.empty(length, 256, dtype=torch.float16, device="cuda")
+    out, _ = model(ids[0], length, 48, spi, spi_t, ppi_t, pp_t, token_type_ids=torch.zeros_like(pos),
+                   position_ids=pos, intermediate_temp=inter)
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    err = (out.float().cpu() - want).abs().max().item()
+    say("  checkpoint err", err)
+    assert err <= 2e-2
+    with pytest.raises(ValueError):
+        bad = json.loads(cfg.to_json_string())
+        bad["hidden_act"] = "relu"
+        (tmp_path / "config.json").write_text(json.dumps(bad))
+        mb.BertModelNoPooler.from_local_checkpoint(str(tmp_path))
