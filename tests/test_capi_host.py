@@ -192,3 +192,19 @@ def test_pipeline_is_race_free_under_thread_sanitizer():
     res = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-4000:]
     assert "pipeline_stress OK" in res.stdout and "ThreadSanitizer" not in res.stderr
+
+
+def test_host_metadata_under_address_and_ub_sanitizers():
+    """meta.cpp built with AddressSanitizer + UndefinedBehaviorSanitizer and driven over random batch
+    geometries with exact-size heap buffers, short capacities and malformed arguments: an out-of-bounds
+    write, a signed overflow or an accepted bad argument makes the run fail."""
+    import subprocess
+    csrc = os.path.join(graft.ROOT, "raptor-t_amd", "csrc")
+    subprocess.check_call(["make", "-C", csrc, "asan_test"], stdout=subprocess.DEVNULL, stderr=subprocess.STDOUT)
+    exe = os.path.join(graft.ROOT, "raptor-t_amd", "build", "meta_fuzz_asan")
+    # the harness preloads a library of its own: AddressSanitizer only checks that its runtime comes first
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=1:exitcode=67",
+               UBSAN_OPTIONS="halt_on_error=1:print_stacktrace=1")
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-4000:]
+    assert "meta_fuzz OK" in res.stdout and "Sanitizer" not in res.stderr
