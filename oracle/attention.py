@@ -79,9 +79,14 @@ def full_attention(q, k, v):
     return torch.matmul(w, v).transpose(0, 1).reshape(length, heads * d)
 
 
-def csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block=64, scale=None):
+def csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block=64, scale=None, seq_tokens=None):
     """q, k, v: [T, H, d] tensors (any float dtype; computed in fp32).  Row of (head h,
-    global from-block g) is `(h if plan_heads > 1 else 0) * NB + g`."""
+    global from-block g) is `(h if plan_heads > 1 else 0) * NB + g`.
+
+    seq_tokens (optional): true token count of each sequence; the positions from there to the end of
+    the sequence's last block are padding and get no attention weight as keys (what the to_mask /
+    band_mask / rand_mask terms of python/modeling_big_bird.py:640-760 do with -10000).  Padded
+    query rows are computed like any other (HuggingFace zeroes them afterwards, :1013)."""
     t, heads, d = q.shape
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     q, k, v = q.float(), k.float(), v.float()
@@ -102,13 +107,17 @@ def csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block=64, sca
                 kk = ks[blocks, :, h].reshape(-1, d)
                 vv = vs[blocks, :, h].reshape(-1, d)
                 qq = q[t0 + i * block: t0 + (i + 1) * block, h]
-                w = torch.softmax(qq @ kk.t() * scale, dim=-1)
+                sc = qq @ kk.t() * scale
+                if seq_tokens is not None:
+                    key_pos = (blocks[:, None] * block + torch.arange(block)[None, :]).reshape(-1)
+                    sc = sc.masked_fill((key_pos >= int(seq_tokens[s]))[None, :], float("-inf"))
+                w = torch.softmax(sc, dim=-1)
                 out[t0 + i * block: t0 + (i + 1) * block, h] = w @ vv
     return out.reshape(t, heads * d)
 
 
-def multiset_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block=64, scale=None):
-    """Brute force in fp64 (small inputs only)."""
+def multiset_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block=64, scale=None, seq_tokens=None):
+    """Brute force in fp64 (small inputs only); seq_tokens as in csr_attention."""
     t, heads, d = q.shape
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     q, k, v = q.double(), k.double(), v.double()
@@ -126,6 +135,8 @@ def multiset_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block=64
                 for j in to_idx[to_pos[row]:to_pos[row + 1]]:
                     count[i, int(j)] += 1.0
             bias = torch.log(count).repeat_interleave(block, 0).repeat_interleave(block, 1)
+            if seq_tokens is not None:
+                bias[:, int(seq_tokens[s]):] = float("-inf")
             sc = q[t0:t0 + length, h] @ k[t0:t0 + length, h].t() * scale + bias
             sc = sc - sc.max(dim=-1, keepdim=True).values
             e = torch.exp(sc)

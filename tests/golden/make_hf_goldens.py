@@ -14,7 +14,8 @@ Outputs (committed, small):
   hf_attention.npz        fp32 outputs of `bigbird_block_sparse_attention` for
                           two tiny single-sequence cases with all-ones masks;
                           the inputs are regenerated from numpy RandomState
-                          seeds recorded in the file.
+                          seeds recorded in the file.  Two more cases carry a padded
+                          tail (attention mask 0 on the last positions).
 The module is put in train() mode because upstream returns an all-zero plan in
 eval mode, a guard the reference deleted.
 """
@@ -59,10 +60,13 @@ def inputs(length, heads, seed):
     return q, k, v
 
 
-def hf_attention(length, heads, seed, in_seed):
+def hf_attention(length, heads, seed, in_seed, tokens=None):
+    """tokens: true length of the sequence; positions from there to `length` are padding (attention mask 0)."""
     m = make_attn(heads, 4096, seed)
     q, k, v = (torch.from_numpy(a)[None] for a in inputs(length, heads, in_seed))
     mask = torch.ones(1, length)
+    if tokens is not None:
+        mask[:, tokens:] = 0.0
     blocked, band, fmask, tmask = BigBirdModel.create_masks_for_block_sparse_attn(mask, 64)
     with torch.no_grad():
         out, _ = m.bigbird_block_sparse_attention(
@@ -89,6 +93,11 @@ def main():
                                                ("L832_H2_seed3", 832, 2, 3, 101)]:
         cases[name + "_out"] = hf_attention(length, heads, seed, in_seed)
         cases[name + "_meta"] = np.array([length, heads, seed, in_seed], dtype=np.int64)
+    # a padded tail: 832 positions of which 800 / 769 are tokens (HuggingFace zeroes the padded query rows)
+    for name, length, heads, seed, in_seed, tokens in [("L832_H2_seed3_len800", 832, 2, 3, 101, 800),
+                                                       ("L1024_H2_seed0_len961", 1024, 2, 0, 100, 961)]:
+        cases[name + "_out"] = hf_attention(length, heads, seed, in_seed, tokens)
+        cases[name + "_meta"] = np.array([length, heads, seed, in_seed, tokens], dtype=np.int64)
     np.savez(os.path.join(HERE, "hf_attention.npz"), **cases)
     print("plans:", len(plans), "attention cases:", [k for k in cases if k.endswith("_out")])
 

@@ -90,3 +90,24 @@ def test_invariants_constant_v_permutation_duplicate_mass():
     e[:, :64] *= 2
     want = (e / e.sum(-1, keepdim=True)) @ v1[:, 0]
     assert (two[:64] - want).abs().max().item() < 1e-5
+
+
+@pytest.mark.parametrize("name", ["L832_H2_seed3_len800", "L1024_H2_seed0_len961"])
+def test_padded_tail_matches_hf_golden(golden_dir, name):
+    """HuggingFace's own masks on a sequence whose last block is partly padding (tests/golden/
+    make_hf_goldens.py) against the oracle's key masking; the padded query rows, which HuggingFace
+    zeroes, are left out.  Masking the wrong side of the boundary, or by block instead of by token,
+    fails this; so does ignoring the mask (checked against the unmasked golden below)."""
+    g = np.load(os.path.join(golden_dir, "hf_attention.npz"))
+    length, heads, seed, in_seed, tokens = (int(x) for x in g[name + "_meta"])
+    want = torch.from_numpy(g[name + "_out"])
+    q, k, v = _inputs(length, heads, in_seed)
+    idx, pos = md.hf_to_index([length], seed, heads)
+    qt, kt, vt = (x.transpose(0, 1).contiguous() for x in (q, k, v))
+    got = oa.csr_attention(qt, kt, vt, [0, length // 64], idx, pos, heads, seq_tokens=[tokens])
+    assert (got[:tokens] - want[:tokens]).abs().max().item() < 2e-6
+    assert want[tokens:].abs().max().item() == 0.0
+    unmasked = oa.csr_attention(qt, kt, vt, [0, length // 64], idx, pos, heads)
+    assert (unmasked[:tokens] - want[:tokens]).abs().max().item() > 1e-3
+    brute = oa.multiset_attention(qt, kt, vt, [0, length // 64], idx, pos, heads, seq_tokens=[tokens])
+    assert (brute[:tokens].float() - want[:tokens]).abs().max().item() < 2e-5
