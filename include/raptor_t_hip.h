@@ -135,6 +135,18 @@ int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out,
                         const int* from_idx, const int* from_pos, int n_wg,
                         int dtype, void* stream);
 
+/* The same launch for a batch whose sequences end in padding (the reference only takes
+ * lengths that are multiples of 64: python/util.py:36-46; this is the to_mask / band_mask /
+ * rand_mask handling of its oracle, python/modeling_big_bird.py:640-760, for a packed batch).
+ * seq_tokens_dev[s] = true token count of sequence s, in (64 * (n_s - 1), 64 * n_s]; the keys from
+ * there to the end of the sequence's last block get no weight.  Padded QUERY rows are computed
+ * like any other row; the caller drops them.  NULL = no padding (rt_bs_attention_fwd). */
+int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, void* out,
+                               const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
+                               int total_blocks, int heads, const int* to_idx, const int* to_pos,
+                               int plan_heads, const int* from_idx, const int* from_pos, int n_wg,
+                               int dtype, void* stream);
+
 /* Replaces kernels::add_bias_and_layernorm_kernel (layers/kernels/
  * add_bias_and_layernorm.cu:268-285): out = LN(out + bias + residual) * gamma + beta,
  * in place on out[rows, hidden]; hidden a multiple of 8. */

@@ -139,10 +139,10 @@ __device__ inline void load_tile(const T* __restrict__ tile, int lane, typename 
 // state.  kbase / vbase point at block 0 of that (sequence, head); n = blocks in the sequence.
 // The row's block ids are fetched 64 at a time into one register (lane j holds entry j) and
 // handed out with v_readlane: one memory round trip per unit instead of one per key block.
-template <typename T>
+template <typename T, bool MASKED>
 __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __restrict__ vbase,
-                                    const int* __restrict__ row, int first, int step, int cnt, int n, int lane,
-                                    const typename Mma<T>::v8 (&qf)[2][4], State& st) {
+                                    const int* __restrict__ row, int first, int step, int cnt, int n, int tail,
+                                    int lane, const typename Mma<T>::v8 (&qf)[2][4], State& st) {
   typedef typename Mma<T>::v8 v8;
   v8 kf[8], vf[8];
   bool fresh = true;                                  // no reference maximum yet
@@ -157,14 +157,14 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
     const int b = __builtin_amdgcn_readlane(ids, e & 63);
     return b < 0 ? 0 : (b >= n ? n - 1 : b);
   };
-  {
-    const int b = block_of(j);
-    load_tile<T>(kbase + int64_t(b) * 4096, lane, kf);
-    load_tile<T>(vbase + int64_t(b) * 4096, lane, vf);
-  }
+  int bcur = block_of(j);
+  load_tile<T>(kbase + int64_t(bcur) * 4096, lane, kf);
+  load_tile<T>(vbase + int64_t(bcur) * 4096, lane, vf);
   for (; j < hi; j += step) {
     const int jn = j + step;
     const bool more = jn < hi;
+    // keys of the sequence's last block beyond its true length are padding: no weight
+    const bool padded = MASKED && tail < 64 && bcur == n - 1;
     // the last iteration re-requests its own tile: loads stay unconditional, so they keep
     // their place in the instruction stream (a branch would sink them next to their use)
     const int bn = block_of(more ? jn : j);
@@ -180,6 +180,13 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
           for (int e = 0; e < 16; ++e) sc[t][e] = init;
 #pragma unroll
           for (int c = 0; c < 4; ++c) sc[t] = Mma<T>::run(kf[t * 4 + c], qf[nt][c], sc[t]);
+        }
+        if (MASKED && padded) {                         // wave-uniform, at most one tile of a row
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+              if (32 * t + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3) >= tail) sc[t][e] = -INFINITY;
         }
       };
       // exp2 of the (already shifted) scores -> P as the B operand of the second product:
@@ -242,6 +249,7 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
         for (int s = 0; s < 4; ++s) st.o[t][nt] = Mma<T>::run(vf[t * 4 + s], pb[s], st.o[t][nt]);
     }
     fresh = false;
+    bcur = bn;
     __builtin_amdgcn_sched_barrier(0);
     load_tile<T>(vbase + int64_t(bn) * 4096, lane, vf);
     __builtin_amdgcn_sched_barrier(0);
@@ -290,6 +298,7 @@ __device__ inline void store_output(T* __restrict__ out_unit, int64_t row_stride
 
 struct Unit {
   int h, i, n, g0;
+  int tail;               // tokens in the sequence's last block that are real (64: none padded)
 };
 
 template <typename T> struct Args {
@@ -297,6 +306,7 @@ template <typename T> struct Args {
   const int* seq_blocks; int batch, heads, nb_total;
   const int* to_idx; const int* to_pos; int plan_heads;
   const int* from_idx; const int* from_pos;
+  const int* seq_tokens;                 // optional: true token count per sequence (padded tail in its last block)
 };
 
 constexpr int MAX_BATCH = 1024;         // sequences per launch (geometry is kept in LDS)
@@ -307,6 +317,7 @@ struct Geometry {
   int sb[MAX_BATCH + 1];
   int gl[MAX_BATCH + 1];
   int bu[MAX_BATCH + 1];
+  int tail[MAX_BATCH];                  // real tokens in each sequence's last block (64 without padding)
 };
 
 __device__ inline int upper_seq(const int* __restrict__ prefix, int batch, int x) {
@@ -331,7 +342,7 @@ __device__ inline void load_q(const Args<T>& a, const Unit& u, int lane, typenam
 }
 
 // One wave, one unit, all of its key blocks.
-template <typename T>
+template <typename T, bool MASKED>
 __device__ inline void run_solo(const Args<T>& a, const Unit& u, int lane, T* stage) {
   typename Mma<T>::v8 qf[2][4];
   const int row = (a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i;
@@ -341,7 +352,7 @@ __device__ inline void run_solo(const Args<T>& a, const Unit& u, int lane, T* st
   const int64_t base = (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n) * 4096;
   State st;
   state_init(st);
-  stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, lane, qf, st);
+  stream_tiles<T, MASKED>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, u.tail, lane, qf, st);
   float w[2];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
@@ -353,7 +364,7 @@ __device__ inline void run_solo(const Args<T>& a, const Unit& u, int lane, T* st
 }
 
 // Four waves, one unit: wave w streams key blocks w, w+4, ...; tree merge through LDS.
-template <typename T>
+template <typename T, bool MASKED>
 __device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int wave, float* park) {
   typename Mma<T>::v8 qf[2][4];
   const int row = (a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i;
@@ -363,7 +374,7 @@ __device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int
   const int64_t base = (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n) * 4096;
   State st;
   state_init(st);
-  stream_tiles<T>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, lane, qf, st);
+  stream_tiles<T, MASKED>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, u.tail, lane, qf, st);
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) st.l[nt] += __shfl_xor(st.l[nt], 32, 64);
 
@@ -431,7 +442,7 @@ __device__ __host__ inline int bundles_per_head(int n) {
 // hardware; the workgroups of XCD x share the x-th eighth of the global items FIRST (they are
 // the long ones) and then the x-th eighth of the bundles, which covers (nearly) the same
 // (sequence, head) groups, so a group's K/V tiles stay in one L2.
-template <typename T>
+template <typename T, bool MASKED>
 __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
   // 34816 bytes: two parked wave states for the global-row merge, or four output staging tiles
   __shared__ __attribute__((aligned(16))) float park[2 * 68 * 64];
@@ -442,6 +453,14 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
 
   for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
   __syncthreads();
+  for (int i = threadIdx.x; i < a.batch; i += 256) {
+    int t = 64;
+    if (MASKED) {
+      t = a.seq_tokens[i] - 64 * (geo.sb[i + 1] - geo.sb[i] - 1);
+      t = t < 1 ? 1 : (t > 64 ? 64 : t);
+    }
+    geo.tail[i] = t;
+  }
   if (threadIdx.x == 0) {
     int g = 0, b = 0;
     for (int s = 0; s < a.batch; ++s) {
@@ -465,6 +484,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
     Unit u;
     u.g0 = geo.sb[lo];
     u.n = geo.sb[lo + 1] - u.g0;
+    u.tail = geo.tail[lo];
     const int rem = unit - u.g0 * a.heads;
     u.h = rem / u.n;
     u.i = rem - u.h * u.n;
@@ -484,13 +504,13 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       if (ids4[0] < 0 || ids4[0] >= n_units) { ++p; continue; }
       const Unit first = unit_of_flat(ids4[0]);
       if (is_global_row(first)) {
-        run_split4<T>(a, first, lane, wave, park);
+        run_split4<T, MASKED>(a, first, lane, wave, park);
         ++p;
         continue;
       }
       int run = 1;
       while (run < 4 && ids4[run] >= 0 && ids4[run] < n_units && !is_global_row(unit_of_flat(ids4[run]))) ++run;
-      if (wave < run) run_solo<T>(a, unit_of_flat(mine_id), lane, stage);
+      if (wave < run) run_solo<T, MASKED>(a, unit_of_flat(mine_id), lane, stage);
       p += run;
     }
     return;
@@ -508,9 +528,10 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       const int rem = item - geo.gl[s];
       u.g0 = geo.sb[s];
       u.n = geo.sb[s + 1] - u.g0;
+      u.tail = geo.tail[s];
       u.h = rem >> 1;
       u.i = (rem & 1) ? u.n - 1 : 0;
-      run_split4<T>(a, u, lane, wave, park);
+      run_split4<T, MASKED>(a, u, lane, wave, park);
       continue;
     }
     const int item = b_lo + (k - g_cnt);
@@ -518,12 +539,13 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
     const int rem = item - geo.bu[s];
     u.g0 = geo.sb[s];
     u.n = geo.sb[s + 1] - u.g0;
+    u.tail = geo.tail[s];
     const int per_head = bundles_per_head(u.n);
     u.h = rem / per_head;
     const int bundle = rem - u.h * per_head;
     const bool sparse = u.n >= RT_MIN_SPARSE_BLOCKS;
     u.i = (sparse ? 1 : 0) + 4 * bundle + wave;
-    if (u.i <= (sparse ? u.n - 2 : u.n - 1)) run_solo<T>(a, u, lane, stage);
+    if (u.i <= (sparse ? u.n - 2 : u.n - 1)) run_solo<T, MASKED>(a, u, lane, stage);
   }
 }
 
@@ -541,10 +563,11 @@ unsigned plan_free_workgroups() {
 
 }  // namespace
 
-extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out, const int* seq_blocks_dev,
-                                   int batch, int total_blocks, int heads, const int* to_idx, const int* to_pos,
-                                   int plan_heads, const int* from_idx, const int* from_pos, int n_wg, int dtype,
-                                   void* stream) {
+extern "C" int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, void* out,
+                                          const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
+                                          int total_blocks, int heads, const int* to_idx, const int* to_pos,
+                                          int plan_heads, const int* from_idx, const int* from_pos, int n_wg,
+                                          int dtype, void* stream) {
   RT_REQUIRE(q && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1, RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d",
              batch, total_blocks, heads);
@@ -566,14 +589,24 @@ extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt,
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == RT_F16) {
     Args<_Float16> a{(const _Float16*)q, (const _Float16*)k, (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch,
-                     heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos};
-    hipLaunchKernelGGL(bs_attention_kernel<_Float16>, dim3(grid), dim3(256), 0, st, a);
+                     heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev};
+    if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<_Float16, true>), dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((bs_attention_kernel<_Float16, false>), dim3(grid), dim3(256), 0, st, a);
   } else {
     Args<__bf16> a{(const __bf16*)q, (const __bf16*)k, (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads,
-                   total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos};
-    hipLaunchKernelGGL(bs_attention_kernel<__bf16>, dim3(grid), dim3(256), 0, st, a);
+                   total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev};
+    if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<__bf16, true>), dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((bs_attention_kernel<__bf16, false>), dim3(grid), dim3(256), 0, st, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "bs_attention launch failed: %s", hipGetErrorString(e));
   return RT_OK;
+}
+
+extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out, const int* seq_blocks_dev,
+                                   int batch, int total_blocks, int heads, const int* to_idx, const int* to_pos,
+                                   int plan_heads, const int* from_idx, const int* from_pos, int n_wg, int dtype,
+                                   void* stream) {
+  return rt_bs_attention_fwd_masked(q, k, vt, out, seq_blocks_dev, nullptr, batch, total_blocks, heads, to_idx, to_pos,
+                                    plan_heads, from_idx, from_pos, n_wg, dtype, stream);
 }

@@ -227,8 +227,15 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
                       int batch_size, const torch::Tensor& seq_len_info_tensor, const torch::Tensor& from_select_index,
                       const torch::Tensor& from_select_index_position, const int* to_select_index,
                       const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
-                      int head_num, std::map<std::string, float>& info, bool balanced) {
+                      int head_num, std::map<std::string, float>& info, bool balanced, const torch::Tensor& seq_tokens) {
   ScopedGpuTimer timer(info, "attention");
+  const int* tokens = nullptr;
+  if (seq_tokens.defined() && seq_tokens.numel() > 0) {
+    if (!seq_tokens.is_cuda() || !seq_tokens.is_contiguous() || seq_tokens.scalar_type() != torch::kInt32 ||
+        seq_tokens.numel() != batch_size)
+      throw std::invalid_argument("attention_mask must be an int32 GPU tensor with the true token count of each sequence");
+    tokens = seq_tokens.data_ptr<int>();
+  }
   const int* from_idx = nullptr;
   const int* from_pos = nullptr;
   int n_wg = 0;
@@ -241,9 +248,10 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
     from_pos = from_select_index_position.data_ptr<int>();
     n_wg = block_limit;
   }
-  check(rt_bs_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), seq_len_info_tensor.data_ptr<int>(),
-                            batch_size, block_num, head_num, to_select_index, to_select_index_position, plan_heads,
-                            from_idx, from_pos, n_wg, dtype_code(out), current_stream()), "rt_bs_attention_fwd");
+  check(rt_bs_attention_fwd_masked(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                   seq_len_info_tensor.data_ptr<int>(), tokens, batch_size, block_num, head_num,
+                                   to_select_index, to_select_index_position, plan_heads, from_idx, from_pos, n_wg,
+                                   dtype_code(out), current_stream()), "rt_bs_attention_fwd");
 }
 
 }  // namespace kernels

@@ -87,7 +87,10 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
                       int batch_size, const torch::Tensor& seq_len_info_tensor, const torch::Tensor& from_select_index,
                       const torch::Tensor& from_select_index_position, const int* to_select_index,
                       const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
-                      int head_num, std::map<std::string, float>& info, bool balanced);
+                      int head_num, std::map<std::string, float>& info, bool balanced,
+                      const torch::Tensor& seq_tokens = torch::Tensor());
+// seq_tokens (optional, int32 on the GPU, one entry per sequence): true token counts of sequences
+// whose last block ends in padding; the padded keys get no weight.
 
 }  // namespace kernels
 }  // namespace layers

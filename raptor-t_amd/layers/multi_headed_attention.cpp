@@ -55,7 +55,7 @@ void MultiHeadedAttention::FuseGemm012AddBIasTranspose(const torch::Tensor& inpu
                                          head_num_, block_num_, head_size_, info, kernel_fusion);
 }
 
-void MultiHeadedAttention::operator()(const torch::Tensor& input_tensor, const torch::Tensor, const std::string attn_type,
+void MultiHeadedAttention::operator()(const torch::Tensor& input_tensor, const torch::Tensor attention_mask, const std::string attn_type,
                                       torch::Tensor& output, torch::Tensor, const std::vector<int> seq_len_info,
                                       torch::Tensor& seq_len_info_tensor, const int block_limit, const int head_size,
                                       const int block_size, const int d_num,
@@ -100,7 +100,7 @@ void MultiHeadedAttention::operator()(const torch::Tensor& input_tensor, const t
   torch::Tensor attention_out = tensor_set->get_tensor("attention_out");
   kernels::sparse_attention(q_out, k_out, v_out, attention_out, batch_size_, seq_len_info_tensor,
                             from_select_index_tensor, from_select_index_position_tensor, to_idx, to_pos, plan_heads,
-                            block_limit, block_num_, head_num_, info, balanced);
+                            block_limit, block_num_, head_num_, info, balanced, attention_mask);
   semaphore->Release(layer_idx_, stream);
 
   kernels::MatMul(attention_out, false, dense_weight_, false, 1, output, 0, handle_, "Attention Output");

@@ -233,7 +233,7 @@ class BertModelNoPooler:
                                       partition_part_tensor=partition_part_tensor, output_layer_temp=output_layer_temp,
                                       intermediate_temp=intermediate_temp, attention_output=attention_output,
                                       test_info={} if test_info is None else test_info, kernel_fusion=kernel_fusion,
-                                      balanced=balanced)
+                                      balanced=balanced, attention_mask=attention_masks)
         roctx.range_pop()
         return out, test_info
 

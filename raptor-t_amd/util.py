@@ -77,3 +77,54 @@ def uniform_lengths(batch, lo, hi, seed=0, block=64):
     """`batch` lengths uniform in [lo, hi], multiples of 64 (BASELINE configs 3 and 5)."""
     rng = np.random.default_rng(seed)
     return (block * rng.integers(lo // block, hi // block + 1, size=batch)).tolist()
+
+
+def pack_padded_batch(input_ids, attention_mask, token_type_ids=None, block_size=64):
+    """Padded HuggingFace-style batch -> the packed batch the encoder takes.
+
+    input_ids, attention_mask: [B, L] (mask 1 on real tokens, which must be a prefix of each row).  Every
+    sequence keeps its real tokens plus the padding needed to fill its own last 64-token block (the
+    reference only takes lengths that are multiples of 64, python/util.py:36-46).  Returns a dict:
+      input_ids, position_ids, token_type_ids : int32 [T] packed, T = sum(seq_lens)
+      seq_lens   : per-sequence packed length, a multiple of block_size
+      seq_tokens : per-sequence true token count (list) and `seq_tokens_tensor` (int32, on the ids' device):
+                   what the layers take as `attention_mask` so that the padded keys get no weight
+    """
+    if input_ids.dim() != 2 or attention_mask.shape != input_ids.shape:
+        raise ValueError("input_ids and attention_mask must both be [batch, length]")
+    mask = attention_mask.to(torch.int64)
+    tokens = mask.sum(dim=1)
+    b, length = input_ids.shape
+    prefix = (torch.arange(length, device=mask.device)[None, :] < tokens[:, None]).to(torch.int64)
+    if not torch.equal(prefix, (mask != 0).to(torch.int64)):
+        raise ValueError("attention_mask must be 1 on a prefix of each row (right padding)")
+    seq_tokens = [int(x) for x in tokens.tolist()]
+    if min(seq_tokens) < 1:
+        raise ValueError("every sequence needs at least one token")
+    seq_lens = [(n + block_size - 1) // block_size * block_size for n in seq_tokens]
+    pad_to = max(seq_lens)
+    if pad_to > length:                                   # the padded width is not a block multiple itself
+        extra = pad_to - length
+        input_ids = torch.nn.functional.pad(input_ids, (0, extra))
+        if token_type_ids is not None:
+            token_type_ids = torch.nn.functional.pad(token_type_ids, (0, extra))
+    ids, pos, typ = [], [], []
+    for s, n in enumerate(seq_lens):
+        ids.append(input_ids[s, :n])
+        pos.append(torch.arange(n, device=input_ids.device))
+        typ.append(token_type_ids[s, :n] if token_type_ids is not None else torch.zeros_like(ids[-1]))
+    cat = lambda xs: torch.cat(xs).to(torch.int32).contiguous()
+    return {"input_ids": cat(ids), "position_ids": cat(pos), "token_type_ids": cat(typ), "seq_lens": seq_lens,
+            "seq_tokens": seq_tokens,
+            "seq_tokens_tensor": torch.tensor(seq_tokens, dtype=torch.int32, device=input_ids.device)}
+
+
+def unpack_to_padded(packed, seq_lens, seq_tokens, length):
+    """[T, D] packed encoder output -> [B, length, D] with zeros on the padded positions (the padded rows of
+    the packed output are whatever the layers computed for padding tokens and are dropped here)."""
+    out = packed.new_zeros(len(seq_lens), length, packed.shape[1])
+    start = 0
+    for s, (n, real) in enumerate(zip(seq_lens, seq_tokens)):
+        out[s, :real] = packed[start:start + real]
+        start += n
+    return out

@@ -45,8 +45,9 @@ def device_plan(capi, seq_lens, heads, seed=0, mode=None, plan_heads=None, devic
     return sb, idx, pos, ph, dev(sb), dev(idx), dev(pos)
 
 
-def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0):
-    """q, k, v: [T, H, 64] CUDA tensors (q unscaled).  Returns (gpu_out [T, H*64], oracle fp32)."""
+def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0, seq_tokens=None):
+    """q, k, v: [T, H, 64] CUDA tensors (q unscaled).  Returns (gpu_out [T, H*64], oracle fp32).
+    seq_tokens: true token count per sequence when its last block ends in padding."""
     sb, idx, pos, ph, sb_d, idx_d, pos_d = device_plan(capi, seq_lens, heads, seed, mode)
     qs = (q.float() * (LOG2E / 8.0)).to(q.dtype)          # the kernel's softmax is base 2
     qp, kp = pack_heads(qs, sb), pack_heads(k, sb)
@@ -56,9 +57,11 @@ def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0):
     if n_wg:
         fp, fi = capi.partition_lpt(sb, heads, n_wg)
         from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
-    capi.bs_attention_fwd(qp, kp, vp, out, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos)
+    tok_d = None if seq_tokens is None else torch.tensor(seq_tokens, dtype=torch.int32).cuda()
+    capi.bs_attention_fwd(qp, kp, vp, out, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos, tok_d)
     torch.cuda.synchronize()
-    ref = oa.csr_attention(qs.cpu(), k.cpu(), v.cpu(), sb.tolist(), idx, pos, ph, scale=1.0 / LOG2E)
+    ref = oa.csr_attention(qs.cpu(), k.cpu(), v.cpu(), sb.tolist(), idx, pos, ph, scale=1.0 / LOG2E,
+                           seq_tokens=seq_tokens)
     return out, ref
 
 

@@ -208,3 +208,32 @@ def test_host_metadata_under_address_and_ub_sanitizers():
     res = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
     assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-4000:]
     assert "meta_fuzz OK" in res.stdout and "Sanitizer" not in res.stderr
+
+
+def test_padded_batch_adapters_round_trip():
+    """pack_padded_batch keeps each sequence's tokens plus the padding that fills its last block, and
+    unpack_to_padded puts rows back where they came from."""
+    import importlib
+    import torch
+    graft.load_package()
+    ut = importlib.import_module("raptor_t_amd.util")
+    lens = [130, 64, 1]
+    width = 150                                           # not a multiple of 64: rows are widened as needed
+    ids = torch.arange(3 * width).view(3, width) + 1
+    mask = (torch.arange(width)[None, :] < torch.tensor(lens)[:, None]).long()
+    p = ut.pack_padded_batch(ids, mask)
+    assert p["seq_lens"] == [192, 64, 64] and p["seq_tokens"] == lens
+    assert p["input_ids"].dtype == torch.int32 and p["input_ids"].numel() == 320
+    assert p["position_ids"][:192].tolist() == list(range(192)) and p["position_ids"][192] == 0
+    assert p["input_ids"][:130].tolist() == ids[0, :130].tolist()
+    assert p["input_ids"][192:256].tolist() == ids[1, :64].tolist()
+    assert p["seq_tokens_tensor"].tolist() == lens
+    hidden = torch.arange(320 * 2, dtype=torch.float32).view(320, 2)
+    back = ut.unpack_to_padded(hidden, p["seq_lens"], p["seq_tokens"], width)
+    assert back.shape == (3, width, 2)
+    assert torch.equal(back[0, :130], hidden[:130]) and torch.equal(back[2, 0], hidden[256])
+    assert back[0, 130:].abs().sum() == 0 and back[2, 1:].abs().sum() == 0
+    with pytest.raises(ValueError):
+        ut.pack_padded_batch(ids, torch.tensor([[1, 0, 1]]).expand(3, 3)[:, :3].repeat(1, 50))   # holes in the mask
+    with pytest.raises(ValueError):
+        ut.pack_padded_batch(ids, torch.zeros_like(mask))

@@ -163,6 +163,34 @@ def test_attention_config2_full_size_properties(capi):
                            np.array(one_idx), np.array(one_pos), 1, scale=1.0 / lh.LOG2E)
     assert (out[sel, h * 64:(h + 1) * 64].float().cpu() - ref).abs().max().item() <= 2e-2
 
+@pytest.mark.parametrize("dtype,n_wg", [(torch.float16, 0), (torch.bfloat16, 0), (torch.float16, 96)])
+def test_attention_padded_tail_matches_oracle(capi, dtype, n_wg):
+    """Sequences whose last block ends in padding: the keys past the true length get no weight.  Covers a
+    sparse sequence, a full-attention one (below 12 blocks), a tail of a single token, and no padding at all;
+    the padded rows hold large values so that a missed mask shows."""
+    say("attention padded", dtype, n_wg)
+    heads = 4
+    seq_lens = [1024, 320, 832, 768]
+    seq_tokens = [1000, 257, 832, 705]
+    t = sum(seq_lens)
+    g = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(t, heads, 64, generator=g) for _ in range(3))
+    start = 0
+    for n, real in zip(seq_lens, seq_tokens):              # loud padding: a key that would dominate if it counted
+        k[start + real:start + n] = 6.0 * torch.sign(q[start:start + 1])
+        v[start + real:start + n] = 50.0
+        start += n
+    q, k, v = (x.to(dtype).cuda() for x in (q, k, v))
+    out, ref = lh.run_attention(capi, q, k, v, seq_lens, heads, seed=2, n_wg=n_wg, seq_tokens=seq_tokens)
+    tol = 2e-2 if dtype == torch.float16 else 6e-2
+    start = 0
+    for n, real in zip(seq_lens, seq_tokens):              # real query rows only
+        err = (out[start:start + real].float().cpu() - ref[start:start + real]).abs().max().item()
+        assert err <= tol, (n, real, err)
+        start += n
+    assert torch.isfinite(out.float()).all()
+
+
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_gemm_matches_torch(capi, dtype):

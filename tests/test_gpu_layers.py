@@ -199,3 +199,49 @@ def test_local_checkpoint_matches_huggingface_bigbird(mb, ut, tmp_path):
         bad["hidden_act"] = "relu"
         (tmp_path / "config.json").write_text(json.dumps(bad))
         mb.BertModelNoPooler.from_local_checkpoint(str(tmp_path))
+
+
+@pytest.mark.parametrize("length,tokens", [(832, 800), (1024, 961)])
+def test_padded_sequence_matches_huggingface_with_attention_mask(mb, ut, length, tokens):
+    """A right-padded sequence: HuggingFace BigBird with its attention mask against the packed model fed
+    through pack_padded_batch, on the real token rows (HuggingFace and this model both leave values of no
+    meaning on the padded rows).  The padding ids are non-zero so that an unmasked key would change the result."""
+    say("hf padded parity", length, tokens)
+    from transformers import BigBirdConfig, BigBirdModel
+    torch.manual_seed(3)
+    cfg = BigBirdConfig(vocab_size=1000, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        intermediate_size=256, max_position_embeddings=4096, attention_type="block_sparse",
+                        block_size=64, num_random_blocks=3, hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+    hf = BigBirdModel(cfg, add_pooling_layer=False).cuda().train()
+    with torch.no_grad():                                  # sharper attention than N(0, 0.02) weights give
+        for layer in hf.encoder.layer:
+            layer.attention.self.query.weight.mul_(6.0)
+            layer.attention.self.key.weight.mul_(6.0)
+            layer.attention.self.value.weight.mul_(5.0)
+    ids = torch.randint(1, 1000, (1, length), device="cuda")
+    mask = (torch.arange(length, device="cuda")[None, :] < tokens).long()
+    with torch.no_grad():
+        want = hf(input_ids=ids, attention_mask=mask).last_hidden_state[0, :tokens].float().cpu()
+        unmasked = hf(input_ids=ids).last_hidden_state[0, :tokens].float().cpu()
+    assert (want - unmasked).abs().max().item() > 5e-2          # the mask matters for this input
+    model = mb.BertModelNoPooler.from_torch(hf, async_=True, dtype=torch.float16)
+    p = ut.pack_padded_batch(ids, mask)
+    assert p["seq_lens"] == [length]
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(p["seq_lens"], 64, 48, 2)
+    meta.update_meta_data(length, spi[-1] + 1, total_comp, spi)
+    inter = torch.empty(length, 256, dtype=torch.float16, device="cuda")
+    for balanced in (True, False):
+        out, _ = model(p["input_ids"], length, 48, spi, spi_t, ppi_t, pp_t, attention_masks=p["seq_tokens_tensor"],
+                       token_type_ids=p["token_type_ids"], position_ids=p["position_ids"], intermediate_temp=inter,
+                       balanced=balanced)
+        torch.cuda.synchronize()
+        got = ut.unpack_to_padded(out, p["seq_lens"], p["seq_tokens"], length)[0, :tokens].float().cpu()
+        err = (got - want).abs().max().item()
+        say("  hf padded err", err)
+        assert err <= 2e-2
+    meta.terminate_thread()
+    with pytest.raises((ValueError, RuntimeError)):
+        model(p["input_ids"], length, 48, spi, spi_t, ppi_t, pp_t, attention_masks=mask.float(),
+              token_type_ids=p["token_type_ids"], position_ids=p["position_ids"], intermediate_temp=inter)
