@@ -88,14 +88,13 @@ template <> struct Mma<__bf16> {
   typedef bf16x8 v8;
   typedef bf16x4 v4;
   __device__ static f32x16 run(v8 a, v8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  // a[0..7] = p[0..7] rounded to bf16; returns the fp32 sum of the UNROUNDED values: converting the
+  // rounded ones back would cost as many instructions again, and the rounding errors of a row's
+  // sum (relative 2^-9 each, random sign) are far below what bf16 outputs resolve
   __device__ static float pack(const float* p, v8& out) {
-    float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      out[e] = static_cast<__bf16>(p[e]);
-      s += static_cast<float>(out[e]);
-    }
-    return s;
+    for (int e = 0; e < 8; ++e) out[e] = static_cast<__bf16>(p[e]);
+    return ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
   }
   __device__ static uint32_t max_bits(const v8& p, uint32_t acc) {
     const u32x4 w = __builtin_bit_cast(u32x4, p);
