@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|ref_e2e]
 
-Default workload `c3` is BASELINE.json's config 3: the 12-layer BigBird-base fp16 encoder
+Default workload `c3` is the headline configuration (benchmark config 3): the 12-layer BigBird-base fp16 encoder
 on a padding-free batch of 16 sequences with lengths uniform in [512, 4096] (multiples of
 64, numpy default_rng(0)), random-init N(0, 0.02) weights, N(0, 1) inputs, driven through
 the drop-in layer API (`raptor_t` pybind module) with the asynchronous metadata pipeline.
@@ -186,7 +186,7 @@ def time_kernel(fn, steps, warmup):
 
 
 def run_attention_only(args):
-    """BASELINE config 2: isolated block-sparse attention, batch 8 x 4096 tokens, 12 heads, fp16."""
+    """Benchmark config 2: isolated block-sparse attention, batch 8 x 4096 tokens, 12 heads, fp16."""
     capi = graft.load_package().capi
     heads, lens = 12, [4096] * 8
     t = sum(lens)
@@ -219,7 +219,7 @@ def run_attention_only(args):
 
 
 def run_membound_sweep(args):
-    """BASELINE config 4: LayerNorm and GELU epilogues over tokens {8K, 32K, 64K}, fp16 and bf16."""
+    """Benchmark config 4: LayerNorm and GELU epilogues over tokens {8K, 32K, 64K}, fp16 and bf16."""
     capi = graft.load_package().capi
     rows = []
     for dt, name in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
@@ -266,8 +266,8 @@ def main():
     ap.add_argument("--cpu-sample-seqs", type=int, default=2)
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (every sequence is independent; see DESIGN.md for how the batch "
-              "would shard); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU (every sequence is independent: a batch would shard over GPUs by "
+              "sequence, with no exchange); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)

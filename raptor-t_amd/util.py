@@ -74,7 +74,7 @@ def generate_input_data(batch_size, seq_lens, vocab=30000, rng=None):
 
 
 def uniform_lengths(batch, lo, hi, seed=0, block=64):
-    """`batch` lengths uniform in [lo, hi], multiples of 64 (BASELINE configs 3 and 5)."""
+    """`batch` lengths uniform in [lo, hi], multiples of 64 (benchmark configs 3 and 5)."""
     rng = np.random.default_rng(seed)
     return (block * rng.integers(lo // block, hi // block + 1, size=batch)).tolist()
 

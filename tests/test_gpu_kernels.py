@@ -126,7 +126,7 @@ def test_attention_large_logits_and_constant_v(capi):
 
 
 def test_attention_config2_full_size_properties(capi):
-    """BASELINE config 2 (batch 8 x 4096 tokens, 12 heads, fp16): too big for the CPU oracle, so
+    """Benchmark config 2 (batch 8 x 4096 tokens, 12 heads, fp16): too big for the CPU oracle, so
     check what the mathematics fixes: global rows equal dense SDPA over the sequence, a
     sample of sparse rows equals the oracle on that one (sequence, head), balanced == unbalanced."""
     say("attention config 2")
