@@ -423,8 +423,12 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
                                                              int batch, int heads, float q_scale) {
   constexpr int N = Vec<T>::N;              // elements per 16 bytes
   constexpr int CPR = 64 / N;               // 16-byte chunks per 64-wide row
-  __shared__ float tile[3][64][65];
-  const int g = blockIdx.x, h = blockIdx.y;
+  // Only V needs a transpose.  A Q / K fragment entry (8 consecutive d of one token) is a run of the
+  // source row already: those two matrices are copied run by run to their permuted places.
+  __shared__ float vtile[64][65];
+  // heads vary fastest over the grid: workgroups running together read neighbouring 128-byte
+  // pieces of the same token rows
+  const int g = blockIdx.y, h = blockIdx.x;
   const int s = find_seq(seq_blocks, batch, g);
   const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
   const int64_t base = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
@@ -432,15 +436,24 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
   const T* src = qkv + int64_t(g) * 64 * (3 * dm) + h * 64;
   for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
     const int row = c / CPR, col = (c % CPR) * N;
+    float x[3][N], b[3][N];
 #pragma unroll
     for (int m = 0; m < 3; ++m) {
-      float x[N], b[N];
-      Vec<T>::load(src + int64_t(row) * 3 * dm + m * dm + col, x);
-      Vec<T>::load(bias + m * dm + h * 64 + col, b);
-      const float sc = m == 0 ? q_scale : 1.0f;
-#pragma unroll
-      for (int i = 0; i < N; ++i) tile[m][row][col + i] = (x[i] + b[i]) * sc;
+      Vec<T>::load(src + int64_t(row) * 3 * dm + m * dm + col, x[m]);
+      Vec<T>::load(bias + m * dm + h * 64 + col, b[m]);
     }
+    // run `col8` (8 elements) of token `row` is lane (row & 31) + 32 * (col8 & 1) of fragment
+    // 4 * (row >> 5) + (col8 >> 1); a 16-byte chunk of fp32 is half such a run
+    const int col8 = col >> 3;
+    const int dst = ((4 * (row >> 5) + (col8 >> 1)) * 64 + (row & 31) + 32 * (col8 & 1)) * 8 + (col & 7);
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      x[0][i] = (x[0][i] + b[0][i]) * q_scale;
+      x[1][i] = x[1][i] + b[1][i];
+      vtile[row][col + i] = x[2][i] + b[2][i];
+    }
+    Vec<T>::store(q + base + dst, x[0]);
+    Vec<T>::store(k + base + dst, x[1]);
   }
   __syncthreads();
   for (int c = threadIdx.x; c < 512; c += 256) {
@@ -448,13 +461,7 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
     const int r32 = 32 * (f >> 2) + (l & 31), c8 = 16 * (f & 3) + 8 * (l >> 5);
     float x[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = tile[0][r32][c8 + e];
-    store8<T>(q + base + c * 8, x);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = tile[1][r32][c8 + e];
-    store8<T>(k + base + c * 8, x);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = tile[2][slot_token(c8 + e)][r32];
+    for (int e = 0; e < 8; ++e) x[e] = vtile[slot_token(c8 + e)][r32];
     store8<T>(vt + base + c * 8, x);
   }
 }
@@ -538,13 +545,13 @@ int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt, const int* seq_blocks_dev,
                       int batch, int total_blocks, int heads, float q_scale, int dtype, void* stream) {
   RT_REQUIRE(qkv && bias && q && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");
-  RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && heads <= 65535, RT_EINVAL,
-             "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
+  RT_REQUIRE(batch >= 1 && total_blocks >= batch && total_blocks <= 65535 && heads >= 1, RT_EINVAL,
+             "bad geometry: batch=%d total_blocks=%d (at most 65535) heads=%d", batch, total_blocks, heads);
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
   RT_REQUIRE(aligned16(qkv) && aligned16(bias) && aligned16(q) && aligned16(k) && aligned16(vt), RT_EINVAL,
              "pointers must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  dim3 grid(total_blocks, heads);
+  dim3 grid(heads, total_blocks);
   if (dtype == RT_F16)
     hipLaunchKernelGGL(qkv_bias_split_kernel<__half>, grid, dim3(256), 0, st, (const __half*)qkv, (const __half*)bias,
                        (__half*)q, (__half*)k, (__half*)vt, seq_blocks_dev, batch, heads, q_scale);
