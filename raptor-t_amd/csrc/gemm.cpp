@@ -86,6 +86,25 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int 
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.la, t, n, k, n));
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.lb, t, k, m, k));
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.lc, t, n, m, n));
+  // A packed batch changes M with every batch.  Once a (N, K, dtype, epilogue) has a winner, a new M
+  // takes it by its index, without asking the heuristic again (cheaper on the host, and the winner of
+  // an exhaustive search need not be among the heuristic's suggestions).
+  {
+    auto known = ctx->tuned_index.find(std::make_tuple(n, k, dtype, epilogue));
+    if (known != ctx->tuned_index.end()) {
+      std::vector<int> index{known->second};
+      std::vector<hipblasLtMatmulHeuristicResult_t> byindex;
+      const float one = 1.0f, zero = 0.0f;
+      size_t ws = 0;
+      if (hipblaslt_ext::getAlgosFromIndex(ctx->lt, index, byindex) == HIPBLAS_STATUS_SUCCESS && !byindex.empty() &&
+          hipblaslt_ext::matmulIsAlgoSupported(ctx->lt, p.desc, &one, p.la, p.lb, &zero, p.lc, p.lc, byindex[0].algo, ws) ==
+              HIPBLAS_STATUS_SUCCESS && ws <= ctx->workspace_bytes) {
+        p.algo = byindex[0].algo;
+        p.ws = ws;
+        return RT_OK;
+      }
+    }
+  }
   hipblasLtMatmulPreference_t pref = nullptr;
   LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
   LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ctx->workspace_bytes,
@@ -124,20 +143,6 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int 
   if (tuned != ctx->tuned_index.end())
     for (int i = 0; i < found && best < 0; ++i)
       if (res[i].state == HIPBLAS_STATUS_SUCCESS && hipblaslt_ext::getIndexFromAlgo(res[i].algo) == tuned->second) best = i;
-  if (best < 0 && tuned != ctx->tuned_index.end()) {
-    // the winner of an exhaustive search need not be among the heuristic's suggestions for this M
-    std::vector<int> index{tuned->second};
-    std::vector<hipblasLtMatmulHeuristicResult_t> byindex;
-    const float one = 1.0f, zero = 0.0f;
-    size_t ws = 0;
-    if (hipblaslt_ext::getAlgosFromIndex(ctx->lt, index, byindex) == HIPBLAS_STATUS_SUCCESS && !byindex.empty() &&
-        hipblaslt_ext::matmulIsAlgoSupported(ctx->lt, p.desc, &one, p.la, p.lb, &zero, p.lc, p.lc, byindex[0].algo, ws) ==
-            HIPBLAS_STATUS_SUCCESS && ws <= ctx->workspace_bytes) {
-      p.algo = byindex[0].algo;
-      p.ws = ws;
-      return RT_OK;
-    }
-  }
   if (best >= 0) {
     p.algo = res[best].algo;
     p.ws = res[best].workspaceSize;
