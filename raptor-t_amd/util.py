@@ -37,8 +37,12 @@ def generate_data_metainfo(input_datas, block_size, thread_block_limit, head_num
     sb = capi.seq_prefix_blocks(lens)
     _, total = capi.block_costs(sb)
     pos, ids = capi.partition_lpt(sb, head_num, thread_block_limit)
-    return (sb.tolist(), torch.from_numpy(sb).to(device), int(total),
-            torch.from_numpy(pos).to(device), torch.from_numpy(ids).to(device))
+    # pinned staging + asynchronous copies: a pageable copy is ordered behind everything already on the
+    # stream and would make the host wait for the previous batch's layers
+    up = lambda a: torch.from_numpy(a).pin_memory().to(device, non_blocking=True)
+    if not str(device).startswith("cuda"):
+        up = lambda a: torch.from_numpy(a).to(device)
+    return sb.tolist(), up(sb), int(total), up(pos), up(ids)
 
 
 def generate_array_with_avg(seq_len, batch_size, max_len, rng=None):
