@@ -36,19 +36,19 @@ def pack_heads(x, seq_blocks, transpose_v=False):
     return torch.cat(parts)
 
 
-def device_plan(capi, seq_lens, heads, seed=0, mode=None, plan_heads=None, device="cuda"):
+def device_plan(capi, seq_lens, heads, seed=0, mode=None, plan_heads=None, device="cuda", max_pos=4096):
     sb = capi.seq_prefix_blocks(seq_lens)
     mode = capi.RT_PLAN_HF if mode is None else mode
     ph = (1 if mode == capi.RT_PLAN_REFERENCE else heads) if plan_heads is None else plan_heads
-    idx, pos = capi.build_to_index(sb, ph, mode=mode, seed=seed)
+    idx, pos = capi.build_to_index(sb, ph, mode=mode, seed=seed, max_pos=max_pos)
     dev = lambda a: torch.from_numpy(a).to(device)
     return sb, idx, pos, ph, dev(sb), dev(idx), dev(pos)
 
 
-def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0, seq_tokens=None):
+def run_attention(capi, q, k, v, seq_lens, heads, seed=0, mode=None, n_wg=0, seq_tokens=None, max_pos=4096):
     """q, k, v: [T, H, 64] CUDA tensors (q unscaled).  Returns (gpu_out [T, H*64], oracle fp32).
     seq_tokens: true token count per sequence when its last block ends in padding."""
-    sb, idx, pos, ph, sb_d, idx_d, pos_d = device_plan(capi, seq_lens, heads, seed, mode)
+    sb, idx, pos, ph, sb_d, idx_d, pos_d = device_plan(capi, seq_lens, heads, seed, mode, max_pos=max_pos)
     qs = (q.float() * (LOG2E / 8.0)).to(q.dtype)          # the kernel's softmax is base 2
     qp, kp = pack_heads(qs, sb), pack_heads(k, sb)
     vp = pack_heads(v, sb, transpose_v=True)

@@ -100,6 +100,21 @@ def test_attention_matches_oracle(capi, dtype, lens, heads, n_wg):
     assert (out.float().cpu() - ref).abs().max().item() <= TOL[dtype]
 
 
+@pytest.mark.parametrize("n_wg", [0, 37])
+def test_attention_rows_longer_than_64_blocks(capi, n_wg):
+    """Sequences beyond 4096 tokens (the BigBird-large configuration goes to 16384): the two global rows
+    list more than 64 key blocks, which the kernel walks in chunks of 64 ids, also when four waves share
+    the row; 65 blocks puts a single entry into the second chunk."""
+    say("attention long rows", n_wg)
+    lens, heads = [8192, 4160, 768], 2
+    t = sum(lens)
+    g = torch.Generator().manual_seed(21)
+    q, k, v = (torch.randn(t, heads, 64, generator=g).half().cuda() for _ in range(3))
+    out, ref = lh.run_attention(capi, q, k, v, lens, heads, seed=4, n_wg=n_wg, max_pos=16384)
+    assert not torch.isnan(out).any()
+    assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
+
+
 def test_attention_reference_plan_shared_heads(capi):
     say("attention reference plan")
     lens, heads = [1024, 1536], 4
