@@ -45,16 +45,17 @@ template <> struct Vec<__hip_bfloat16> {
 #pragma unroll
     for (int i = 0; i < 4; ++i) { f[2 * i] = __uint_as_float(w[i] << 16); f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
   }
-  __device__ static uint32_t rne(float x) {          // float -> bf16 bits, round to nearest even
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;   // keep NaN a NaN
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  // float pair -> packed bf16, round to nearest even: one v_cvt_pk_bf16_f32 on gfx950
+  __device__ static uint32_t pack2(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 h = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, h);
   }
   __device__ static void store(__hip_bfloat16* p, const float* f) {
     uint4 r;
     uint32_t* w = reinterpret_cast<uint32_t*>(&r);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) w[i] = rne(f[2 * i]) | (rne(f[2 * i + 1]) << 16);
+    for (int i = 0; i < 4; ++i) w[i] = pack2(f[2 * i], f[2 * i + 1]);
     *reinterpret_cast<uint4*>(p) = r;
   }
 };
@@ -427,8 +428,10 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
   // source row already: those two matrices are copied run by run to their permuted places.
   __shared__ float vtile[64][65];
   // heads vary fastest over the grid: workgroups running together read neighbouring 128-byte
-  // pieces of the same token rows
-  const int g = blockIdx.y, h = blockIdx.x;
+  // pieces of the same token rows.  The head is rotated by the block index so that, with a
+  // power-of-two head count, one XCD (workgroups go to the 8 XCDs round-robin) does not always get
+  // the same heads' columns.
+  const int g = blockIdx.x / heads, h = (blockIdx.x % heads + g) % heads;
   const int s = find_seq(seq_blocks, batch, g);
   const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
   const int64_t base = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
@@ -545,13 +548,13 @@ int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt, const int* seq_blocks_dev,
                       int batch, int total_blocks, int heads, float q_scale, int dtype, void* stream) {
   RT_REQUIRE(qkv && bias && q && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");
-  RT_REQUIRE(batch >= 1 && total_blocks >= batch && total_blocks <= 65535 && heads >= 1, RT_EINVAL,
-             "bad geometry: batch=%d total_blocks=%d (at most 65535) heads=%d", batch, total_blocks, heads);
+  RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && int64_t(total_blocks) * heads < (int64_t(1) << 31),
+             RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
   RT_REQUIRE(aligned16(qkv) && aligned16(bias) && aligned16(q) && aligned16(k) && aligned16(vt), RT_EINVAL,
              "pointers must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  dim3 grid(heads, total_blocks);
+  dim3 grid(unsigned(heads) * unsigned(total_blocks));
   if (dtype == RT_F16)
     hipLaunchKernelGGL(qkv_bias_split_kernel<__half>, grid, dim3(256), 0, st, (const __half*)qkv, (const __half*)bias,
                        (__half*)q, (__half*)k, (__half*)vt, seq_blocks_dev, batch, heads, q_scale);
