@@ -115,6 +115,23 @@ def test_attention_rows_longer_than_64_blocks(capi, n_wg):
     assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
 
 
+def test_attention_maximum_batch(capi):
+    """1024 sequences in one launch is the limit of the kernel's LDS geometry tables; one more is refused."""
+    say("attention max batch")
+    heads = 1
+    lens = [64] * 1000 + [128] * 24
+    t = sum(lens)
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(t, heads, 64, generator=g).half().cuda() for _ in range(3))
+    out, ref = lh.run_attention(capi, q, k, v, lens, heads, seed=0)
+    assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
+    lens = [64] * 1025
+    t = sum(lens)
+    q, k, v = (torch.zeros(t, heads, 64).half().cuda() for _ in range(3))
+    with pytest.raises(capi.RaptorError):
+        lh.run_attention(capi, q, k, v, lens, heads, seed=0)
+
+
 def test_attention_reference_plan_shared_heads(capi):
     say("attention reference plan")
     lens, heads = [1024, 1536], 4
