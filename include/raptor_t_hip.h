@@ -179,7 +179,7 @@ int rt_gemm_create(rt_gemm_ctx** ctx);
 int rt_gemm_destroy(rt_gemm_ctx* ctx);
 /* How many hipBLASLt heuristic candidates are timed (once per (N, K, dtype, epilogue), on the
  * operands of the first rt_gemm call of that kind) before one is kept: 1 = take the library's
- * first suggestion, default 16; RT_GEMM_TUNE_ALL = every solution of the library that accepts
+ * first suggestion, default 64 (about 40 ms per kind); RT_GEMM_TUNE_ALL = every solution of the library that accepts
  * the problem (seconds per kind, once per process). */
 #define RT_GEMM_TUNE_ALL (-1)
 int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates);
@@ -194,6 +194,14 @@ int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c,
 enum { RT_EPILOGUE_NONE = 0, RT_EPILOGUE_BIAS = 1, RT_EPILOGUE_BIAS_GELU = 2 };
 int rt_gemm_bias_act(rt_gemm_ctx* ctx, const void* a, const void* b, const void* bias, void* c,
                      int64_t m, int64_t n, int64_t k, int epilogue, int dtype, void* stream);
+
+/* C[M,N] = A[M,K] . Bt[N,K]^T with any of the three epilogues (bias may be NULL for
+ * RT_EPILOGUE_NONE): the b_trans = true form of kernels::MatMul
+ * (layers/kernels/mat_mul.cpp:9-96, which passes CUBLAS_OP_T for it).  Both operands are then
+ * contiguous along K, the layout the library's kernels for these shapes are fastest on, so the
+ * layer objects keep their weights as [out, in] and call this. */
+int rt_gemm_bt(rt_gemm_ctx* ctx, const void* a, const void* bt, const void* bias, void* c,
+               int64_t m, int64_t n, int64_t k, int epilogue, int dtype, void* stream);
 
 /* ------------------------------------------------------- metadata / stream pipeline */
 

@@ -25,7 +25,7 @@ EXPORTS = [
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm",
-    "rt_gemm_bias_act",
+    "rt_gemm_bias_act", "rt_gemm_bt",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
 ]
@@ -69,6 +69,7 @@ def lib():
         L.rt_gemm.argtypes = [vp, vp, vp, vp, L64, L64, L64, I, vp]
         L.rt_embed_layernorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, L64, I, I, I, I, ctypes.c_float, I, I, vp]
         L.rt_gemm_bias_act.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
+        L.rt_gemm_bt.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
         L.rt_pipeline_create.argtypes = [ctypes.POINTER(vp), I, I, I, I, I, I, I]
         L.rt_pipeline_publish.argtypes = [vp, i32p, I]
         L.rt_pipeline_acquire.argtypes = [vp, I, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), i32p,
@@ -251,6 +252,14 @@ class Gemm:
         n = b.shape[1]
         check(lib().rt_gemm_bias_act(self._h, _dp(a), _dp(b), _dp(bias), _dp(c), m, n, k, epilogue, _dtype_code(a),
                                      _stream()))
+        return c
+
+    def bt(self, a, bt, c, bias=None, epilogue=RT_EPILOGUE_NONE):
+        """c = a @ bt.T (+ bias, + GELU as `epilogue` says) with the weights kept as bt[N, K]."""
+        m, k = a.shape
+        n = bt.shape[0]
+        check(lib().rt_gemm_bt(self._h, _dp(a), _dp(bt), None if bias is None else _dp(bias), _dp(c), m, n, k, epilogue,
+                               _dtype_code(a), _stream()))
         return c
 
     def close(self):

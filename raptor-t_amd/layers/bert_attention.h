@@ -17,7 +17,7 @@ class BertAttention : public MultiHeadedAttention {
                              std::move(qkv_bias), std::move(layer_norm_weight), std::move(layer_norm_bias),
                              num_attention_heads, layer_idx, async, layer_norm_eps) {
     head_num_ = num_attention_heads;
-    d_num_ = qkv_weight_.size(0);
+    d_num_ = qkv_weight_.size(1);   // stored as [3D, D]
     block_size_ = RT_BLOCK;
     head_size_ = d_num_ / head_num_;
   }

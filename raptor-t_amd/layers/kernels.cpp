@@ -117,17 +117,23 @@ ScopedGpuTimer::~ScopedGpuTimer() {
 
 void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b_trans, float alpha,
             torch::Tensor& out, float beta, rt_gemm_ctx* handle, const std::string& name) {
-  if (a_trans || b_trans || alpha != 1.0f || beta != 0.0f)
-    throw std::invalid_argument(name + ": only out = A . B is supported");
+  if (a_trans || alpha != 1.0f || beta != 0.0f)
+    throw std::invalid_argument(name + ": only out = A . B and out = A . B^T are supported");
   require_cuda_contiguous(A, "A");
   require_cuda_contiguous(B, "B");
   require_cuda_contiguous(out, "out");
-  if (A.dim() != 2 || B.dim() != 2 || A.size(1) != B.size(0) || out.numel() != A.size(0) * B.size(1))
+  if (A.dim() != 2 || B.dim() != 2) throw std::invalid_argument(name + ": operands must be matrices");
+  const int64_t n = b_trans ? B.size(0) : B.size(1);
+  if (A.size(1) != (b_trans ? B.size(1) : B.size(0)) || out.numel() != A.size(0) * n)
     throw std::invalid_argument(name + ": shape mismatch");
   static std::map<std::string, float> no_info;
   ScopedGpuTimer timer(no_info, "MatMul");
-  check(rt_gemm(handle, A.data_ptr(), B.data_ptr(), out.data_ptr(), A.size(0), B.size(1), A.size(1), dtype_code(A),
-                current_stream()), name.c_str());
+  if (b_trans)
+    check(rt_gemm_bt(handle, A.data_ptr(), B.data_ptr(), nullptr, out.data_ptr(), A.size(0), n, A.size(1),
+                     RT_EPILOGUE_NONE, dtype_code(A), current_stream()), name.c_str());
+  else
+    check(rt_gemm(handle, A.data_ptr(), B.data_ptr(), out.data_ptr(), A.size(0), n, A.size(1), dtype_code(A),
+                  current_stream()), name.c_str());
 }
 
 namespace {
@@ -137,17 +143,23 @@ void set_gemm_epilogue_fusion(bool on) { g_epilogue_fusion.store(on); }
 bool gemm_epilogue_fusion() { return g_epilogue_fusion.load(); }
 
 void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch::Tensor& bias, torch::Tensor& out,
-                    rt_gemm_ctx* handle, std::map<std::string, float>& info, const std::string& name) {
+                    rt_gemm_ctx* handle, std::map<std::string, float>& info, const std::string& name, bool b_trans) {
   require_cuda_contiguous(A, "A");
   require_cuda_contiguous(B, "B");
   require_cuda_contiguous(bias, "bias");
   require_cuda_contiguous(out, "out");
-  if (A.dim() != 2 || B.dim() != 2 || A.size(1) != B.size(0) || out.numel() != A.size(0) * B.size(1) ||
-      bias.numel() != B.size(1) || bias.scalar_type() != A.scalar_type())
+  if (A.dim() != 2 || B.dim() != 2) throw std::invalid_argument(name + ": operands must be matrices");
+  const int64_t n = b_trans ? B.size(0) : B.size(1);
+  if (A.size(1) != (b_trans ? B.size(1) : B.size(0)) || out.numel() != A.size(0) * n || bias.numel() != n ||
+      bias.scalar_type() != A.scalar_type())
     throw std::invalid_argument(name + ": shape or dtype mismatch");
   ScopedGpuTimer timer(info, "MatMul_bias_gelu");
-  check(rt_gemm_bias_act(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), B.size(1),
-                         A.size(1), RT_EPILOGUE_BIAS_GELU, dtype_code(A), current_stream()), name.c_str());
+  if (b_trans)
+    check(rt_gemm_bt(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), n, A.size(1),
+                     RT_EPILOGUE_BIAS_GELU, dtype_code(A), current_stream()), name.c_str());
+  else
+    check(rt_gemm_bias_act(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), n, A.size(1),
+                           RT_EPILOGUE_BIAS_GELU, dtype_code(A), current_stream()), name.c_str());
 }
 
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,

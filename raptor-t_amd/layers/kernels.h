@@ -51,8 +51,9 @@ class ScopedGpuTimer {
   void* stop_ = nullptr;
 };
 
-// kernels::MatMul (layers/kernels/mat_mul.cpp:9-96): out[M,N] = A[M,K] . B[K,N]; only the
-// no-transpose, alpha = 1, beta = 0 form the layers use is supported.
+// kernels::MatMul (layers/kernels/mat_mul.cpp:9-96): out[M,N] = A[M,K] . B[K,N], or
+// A[M,K] . B[N,K]^T with b_trans (the faster layout here: both operands contiguous along K);
+// a_trans, alpha != 1 and beta != 0, which no layer uses, are refused.
 void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b_trans, float alpha,
             torch::Tensor& out, float beta, rt_gemm_ctx* handle, const std::string& name);
 
@@ -60,7 +61,8 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
 // its epilogue (what BertIntermediate's pair of calls, layers/bert_intermediate.cpp:22-30,
 // computes).  Times itself under "MatMul_bias_gelu".
 void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch::Tensor& bias, torch::Tensor& out,
-                    rt_gemm_ctx* handle, std::map<std::string, float>& info, const std::string& name);
+                    rt_gemm_ctx* handle, std::map<std::string, float>& info, const std::string& name,
+                    bool b_trans = false);
 // Whether BertIntermediate uses MatMulBiasGelu when kernel_fusion is asked for (default) or
 // keeps the GEMM and the bias + GELU kernel apart.
 void set_gemm_epilogue_fusion(bool on);

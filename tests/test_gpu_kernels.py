@@ -322,6 +322,40 @@ def test_gemm_bias_gelu_epilogue_matches_oracle(capi, dtype):
     gemm.close()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_gemm_transposed_weights_match_plain(capi, dtype):
+    """rt_gemm_bt (weights kept as [N, K]) against an fp64 product and against rt_gemm / rt_gemm_bias_act on the
+    [K, N] copy of the same weights, for each epilogue."""
+    say("gemm bt", dtype)
+    g = torch.Generator().manual_seed(4)
+    gemm = capi.Gemm()
+    for m, n, k in [(832, 2304, 768), (200, 768, 3072), (1, 512, 256)]:
+        a = torch.randn(m, k, generator=g).to(dtype).cuda()
+        bt = (torch.randn(n, k, generator=g) * 0.05).to(dtype).cuda()
+        b = bt.t().contiguous()
+        bias = torch.randn(n, generator=g).to(dtype).cuda()
+        prod = a.double().cpu() @ bt.double().cpu().t()
+        tol = (2e-2 if dtype == torch.float16 else 6e-2) if dtype != torch.float32 else 2e-3
+        got, ref = (torch.empty(m, n, dtype=dtype, device="cuda") for _ in range(2))
+        gemm.bt(a, bt, got)
+        gemm(a, b, ref)
+        torch.cuda.synchronize()
+        assert (got.double().cpu() - prod).abs().max().item() <= tol * max(1.0, prod.abs().max().item() / 4)
+        assert (got.float() - ref.float()).abs().max().item() <= tol
+        if dtype == torch.float32:
+            continue                                        # the library has no fp32 bias epilogue for every shape
+        for ep, want in ((capi.RT_EPILOGUE_BIAS, prod + bias.double().cpu()),
+                         (capi.RT_EPILOGUE_BIAS_GELU, ol.bias_gelu(prod, bias.cpu()))):
+            gemm.bt(a, bt, got, bias=bias, epilogue=ep)
+            gemm.bias_act(a, b, bias, ref, ep)
+            torch.cuda.synchronize()
+            assert (got.double().cpu() - want).abs().max().item() <= tol
+            assert (got.float() - ref.float()).abs().max().item() <= tol
+    with pytest.raises(capi.RaptorError):
+        gemm.bt(a, bt, got, bias=None, epilogue=capi.RT_EPILOGUE_BIAS)
+    gemm.close()
+
+
 @pytest.mark.parametrize("dtype,hidden,heads,ffn,n_wg", [
     (torch.float16, 768, 12, 3072, 0), (torch.bfloat16, 1024, 16, 4096, 64), (torch.float16, 768, 12, 3072, 160)])
 def test_encoder_layer_matches_oracle(capi, dtype, hidden, heads, ffn, n_wg):
