@@ -45,7 +45,7 @@ def block_pairs(seq_blocks, heads):
 # what the same counters read for the QKV split kernel (a copy of known size); the summaries and the commands are
 # in profiles/memory_kernels_c3_traffic.txt.  Only valid for that workload.
 MEASURED_TRAFFIC_C3 = {"bs_attention_kernel": 404.0e6, "bias_residual_layernorm_kernel": 171.4e6,
-                       "bias_gelu_kernel": 457.2e6, "qkv_bias_split_kernel": 342.7e6}
+                       "bias_gelu_kernel": 457.2e6, "qkv_bias_split_kernel_q": 342.7e6, "qkv_bias_split_kernel": None}
 
 
 def hbm_roofline(name, bytes_per_launch, us_per_launch, traffic=None):
@@ -107,6 +107,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
             balanced=args.lpt_plan)
 
     mb.cxx.set_gemm_epilogue_fusion(not args.no_epilogue_fusion)
+    mb.cxx.set_attention_q_from_rows(not args.materialize_q)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -150,6 +151,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
                    "batch": len(seq_lens), "tokens": t, "seq_lens": seq_lens, "block_limit": block_limit,
                    "balanced": args.lpt_plan, "async_index": not args.sync_index,
                    "gemm_epilogue_fusion": not args.no_epilogue_fusion,
+                   "attention_q_from_rows": not args.materialize_q,
                    "weights": "random N(0,0.02)", "plan": "per-head HF plan, seed = layer index"},
         "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12,
                      "peak": MFMA_PEAK[dtype] / 1e12, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK[dtype],
@@ -160,8 +162,11 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
                                            traffic.get("bias_residual_layernorm_kernel")),
         "roofline_gelu": dict(hbm_roofline("bias_gelu_kernel", 2 * t * ffn * sz, per["add_bias_act_kernel"],
                                            traffic.get("bias_gelu_kernel")), measured=gelu_note),
-        "roofline_qkv_split": hbm_roofline("qkv_bias_split_kernel", 2 * t * 3 * hidden * sz,
-                                           per["add_bias_and_transpose_kernel"], traffic.get("qkv_bias_split_kernel")),
+        # K and V only (read + write) unless Q is materialised too
+        "roofline_qkv_split": hbm_roofline("qkv_bias_split_kernel", 2 * t * (3 if args.materialize_q else 2) * hidden * sz,
+                                           per["add_bias_and_transpose_kernel"],
+                                           traffic.get("qkv_bias_split_kernel_q" if args.materialize_q
+                                                       else "qkv_bias_split_kernel")),
         "kernel_us_per_launch": per,
         "kernel_us_per_step": {k: v[0] / args.steps for k, v in timing_all.items()},
         "kernel_timing": "attention: HIP events inside the timed steps; the others: a second pass over the same "
@@ -311,6 +316,9 @@ def main():
     ap.add_argument("--sync-index", action="store_true", help="build the block index inline instead of on the workers")
     ap.add_argument("--no-epilogue-fusion", action="store_true",
                     help="keep bias + GELU as its own kernel instead of the intermediate GEMM's epilogue")
+    ap.add_argument("--materialize-q", action="store_true",
+                    help="the split kernel writes Q too and the attention kernel reads it from there (the reference's "
+                         "arrangement) instead of taking its queries from the projection's output rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=2)
     args = ap.parse_args()

@@ -111,7 +111,9 @@ int rt_meta_partition_lpt(const int* seq_blocks, int batch, int heads, int n_wg,
 /* Replaces kernels::add_bias_and_transpose_kernel (layers/kernels/
  * add_bias_and_transpose.cu:212-233): qkv[T, 3*H*64] token-major + bias[3*H*64] ->
  * q (scaled by q_scale), k, vt in the head-major packed layout.  For rt_bs_attention_fwd
- * q_scale must be log2(e)/sqrt(64): the attention kernel evaluates the softmax in base 2. */
+ * q_scale must be log2(e)/sqrt(64): the attention kernel evaluates the softmax in base 2.
+ * q may be NULL: Q is then not written (a third less traffic), for rt_bs_attention_fwd_qrows,
+ * which takes its queries from `qkv` itself. */
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt,
                       const int* seq_blocks_dev, int batch, int total_blocks, int heads,
                       float q_scale, int dtype, void* stream);
@@ -146,6 +148,20 @@ int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, voi
                                int total_blocks, int heads, const int* to_idx, const int* to_pos,
                                int plan_heads, const int* from_idx, const int* from_pos, int n_wg,
                                int dtype, void* stream);
+
+/* The same launch with the queries read where the QKV projection left them: `qkv` is the
+ * [T, 3*H*64] input of rt_qkv_bias_split (columns 0 .. H*64-1 are Q), `qkv_bias` its bias; each
+ * unit adds the bias and applies q_scale to its 64x64 query tile as it loads it (once per unit,
+ * the same fp32 arithmetic and rounding as the split kernel, so both routes give the same bits).
+ * k and vt still come from rt_qkv_bias_split (called with q = NULL).  Same stage of the
+ * reference as rt_bs_attention_fwd; the reference always materialises Q
+ * (layers/kernels/add_bias_and_transpose.cu:212-233).  seq_tokens_dev may be NULL. */
+int rt_bs_attention_fwd_qrows(const void* qkv, const void* qkv_bias, float q_scale, const void* k,
+                              const void* vt, void* out, const int* seq_blocks_dev,
+                              const int* seq_tokens_dev, int batch, int total_blocks, int heads,
+                              const int* to_idx, const int* to_pos, int plan_heads,
+                              const int* from_idx, const int* from_pos, int n_wg, int dtype,
+                              void* stream);
 
 /* Replaces kernels::add_bias_and_layernorm_kernel (layers/kernels/
  * add_bias_and_layernorm.cu:268-285): out = LN(out + bias + residual) * gamma + beta,

@@ -306,6 +306,9 @@ template <typename T> struct Args {
   const int* to_idx; const int* to_pos; int plan_heads;
   const int* from_idx; const int* from_pos;
   const int* seq_tokens;                 // optional: true token count per sequence (padded tail in its last block)
+  // optional: Q taken from the QKV projection's own output rows [tokens, 3 * heads * 64] (columns
+  // 0 .. heads*64-1), bias added and scale applied while loading; q is then unused
+  const T* q_rows; const T* q_bias; float q_scale;
 };
 
 constexpr int MAX_BATCH = 1024;         // sequences per launch (geometry is kept in LDS)
@@ -333,6 +336,24 @@ __device__ inline bool is_global_row(const Unit& u) { return u.n >= RT_MIN_SPARS
 template <typename T>
 __device__ inline void load_q(const Args<T>& a, const Unit& u, int lane, typename Mma<T>::v8 (&qf)[2][4]) {
   typedef typename Mma<T>::v8 v8;
+  if (a.q_rows) {
+    // fragment (nt, c), lane l = dims 16c + 8(l >> 5) .. +7 of query 32nt + (l & 31): a 16-byte run of
+    // the token's row.  Same arithmetic as the split kernel: (x + bias) * scale in fp32, rounded once.
+    const int64_t ld = int64_t(a.heads) * 192;
+    const T* src = a.q_rows + (int64_t(u.g0 + u.i) * 64 + (lane & 31)) * ld + u.h * 64 + (lane >> 5) * 8;
+    const T* bsrc = a.q_bias + u.h * 64 + (lane >> 5) * 8;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const v8 b = *reinterpret_cast<const v8*>(bsrc + c * 16);
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const v8 x = *reinterpret_cast<const v8*>(src + nt * 32 * ld + c * 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[nt][c][e] = static_cast<T>((float(x[e]) + float(b[e])) * a.q_scale);
+      }
+    }
+    return;
+  }
   const T* qt = a.q + (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n + u.i) * 4096;
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt)
@@ -562,20 +583,22 @@ unsigned plan_free_workgroups() {
 
 }  // namespace
 
-extern "C" int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, void* out,
-                                          const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
-                                          int total_blocks, int heads, const int* to_idx, const int* to_pos,
-                                          int plan_heads, const int* from_idx, const int* from_pos, int n_wg,
-                                          int dtype, void* stream) {
-  RT_REQUIRE(q && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
+namespace {
+
+int launch_attention(const void* q, const void* q_rows, const void* q_bias, float q_scale, const void* k, const void* vt,
+                     void* out, const int* seq_blocks_dev, const int* seq_tokens_dev, int batch, int total_blocks,
+                     int heads, const int* to_idx, const int* to_pos, int plan_heads, const int* from_idx,
+                     const int* from_pos, int n_wg, int dtype, void* stream) {
+  RT_REQUIRE((q || (q_rows && q_bias)) && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1, RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d",
              batch, total_blocks, heads);
   RT_REQUIRE(plan_heads == 1 || plan_heads == heads, RT_EINVAL, "plan_heads=%d must be 1 or heads=%d", plan_heads, heads);
   RT_REQUIRE((from_idx == nullptr) == (from_pos == nullptr), RT_EINVAL, "from_idx and from_pos go together");
   RT_REQUIRE(int64_t(total_blocks) * heads < (int64_t(1) << 31), RT_EINVAL, "too many units");
   RT_REQUIRE(batch <= MAX_BATCH, RT_EINVAL, "at most %d sequences per launch, got %d", MAX_BATCH, batch);
-  RT_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(vt) |
-               reinterpret_cast<uintptr_t>(out)) & 15u) == 0, RT_EINVAL, "q, k, vt, out must be 16-byte aligned");
+  RT_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(q_rows) | reinterpret_cast<uintptr_t>(q_bias) |
+               reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(vt) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0,
+             RT_EINVAL, "q (or qkv and its bias), k, vt, out must be 16-byte aligned");
   if (dtype == RT_F32) return rt::fail(RT_ENOSYS, "block-sparse attention runs in fp16 or bf16 (fp32 accumulation)");
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16, RT_EINVAL, "unknown dtype %d", dtype);
   unsigned grid;
@@ -588,18 +611,42 @@ extern "C" int rt_bs_attention_fwd_masked(const void* q, const void* k, const vo
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == RT_F16) {
     Args<_Float16> a{(const _Float16*)q, (const _Float16*)k, (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch,
-                     heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev};
+                     heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
+                     (const _Float16*)q_rows, (const _Float16*)q_bias, q_scale};
     if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<_Float16, true>), dim3(grid), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((bs_attention_kernel<_Float16, false>), dim3(grid), dim3(256), 0, st, a);
   } else {
     Args<__bf16> a{(const __bf16*)q, (const __bf16*)k, (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads,
-                   total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev};
+                   total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
+                   (const __bf16*)q_rows, (const __bf16*)q_bias, q_scale};
     if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<__bf16, true>), dim3(grid), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((bs_attention_kernel<__bf16, false>), dim3(grid), dim3(256), 0, st, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "bs_attention launch failed: %s", hipGetErrorString(e));
   return RT_OK;
+}
+
+}  // namespace
+
+extern "C" int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, void* out,
+                                          const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
+                                          int total_blocks, int heads, const int* to_idx, const int* to_pos,
+                                          int plan_heads, const int* from_idx, const int* from_pos, int n_wg,
+                                          int dtype, void* stream) {
+  RT_REQUIRE(q, RT_EINVAL, "NULL pointer");
+  return launch_attention(q, nullptr, nullptr, 1.0f, k, vt, out, seq_blocks_dev, seq_tokens_dev, batch, total_blocks, heads,
+                          to_idx, to_pos, plan_heads, from_idx, from_pos, n_wg, dtype, stream);
+}
+
+extern "C" int rt_bs_attention_fwd_qrows(const void* qkv, const void* qkv_bias, float q_scale, const void* k,
+                                         const void* vt, void* out, const int* seq_blocks_dev,
+                                         const int* seq_tokens_dev, int batch, int total_blocks, int heads,
+                                         const int* to_idx, const int* to_pos, int plan_heads, const int* from_idx,
+                                         const int* from_pos, int n_wg, int dtype, void* stream) {
+  RT_REQUIRE(qkv && qkv_bias, RT_EINVAL, "NULL pointer");
+  return launch_attention(nullptr, qkv, qkv_bias, q_scale, k, vt, out, seq_blocks_dev, seq_tokens_dev, batch, total_blocks,
+                          heads, to_idx, to_pos, plan_heads, from_idx, from_pos, n_wg, dtype, stream);
 }
 
 extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out, const int* seq_blocks_dev,

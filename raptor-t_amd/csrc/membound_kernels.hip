@@ -442,6 +442,7 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
     float x[3][N], b[3][N];
 #pragma unroll
     for (int m = 0; m < 3; ++m) {
+      if (m == 0 && !q) continue;                       // Q is left to the attention kernel
       Vec<T>::load(src + int64_t(row) * 3 * dm + m * dm + col, x[m]);
       Vec<T>::load(bias + m * dm + h * 64 + col, b[m]);
     }
@@ -451,11 +452,11 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
     const int dst = ((4 * (row >> 5) + (col8 >> 1)) * 64 + (row & 31) + 32 * (col8 & 1)) * 8 + (col & 7);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      x[0][i] = (x[0][i] + b[0][i]) * q_scale;
+      if (q) x[0][i] = (x[0][i] + b[0][i]) * q_scale;
       x[1][i] = x[1][i] + b[1][i];
       vtile[row][col + i] = x[2][i] + b[2][i];
     }
-    Vec<T>::store(q + base + dst, x[0]);
+    if (q) Vec<T>::store(q + base + dst, x[0]);
     Vec<T>::store(k + base + dst, x[1]);
   }
   __syncthreads();
@@ -547,7 +548,7 @@ int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype
 
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt, const int* seq_blocks_dev,
                       int batch, int total_blocks, int heads, float q_scale, int dtype, void* stream) {
-  RT_REQUIRE(qkv && bias && q && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(qkv && bias && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");       // q may be NULL: not written
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && int64_t(total_blocks) * heads < (int64_t(1) << 31),
              RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);

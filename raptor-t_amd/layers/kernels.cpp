@@ -138,7 +138,11 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
 
 namespace {
 std::atomic<bool> g_epilogue_fusion{true};
+std::atomic<bool> g_q_from_rows{true};
+constexpr float kQScale = 1.4426950408889634f / 8.0f;      // log2(e) / sqrt(64): the softmax runs in base 2
 }
+void set_attention_q_from_rows(bool on) { g_q_from_rows.store(on); }
+bool attention_q_from_rows() { return g_q_from_rows.load(); }
 void set_gemm_epilogue_fusion(bool on) { g_epilogue_fusion.store(on); }
 bool gemm_epilogue_fusion() { return g_epilogue_fusion.load(); }
 
@@ -169,9 +173,10 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
   ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel");
   if (head_size != RT_HEAD_DIM) throw std::invalid_argument("head size must be 64");
   // the attention kernel evaluates the softmax in base 2: fold log2(e) into the Q scale
-  const float scale = 1.4426950408889634f / std::sqrt(float(head_size));
+  const float scale = kQScale;
   if (kernel_fusion) {
-    check(rt_qkv_bias_split(input_data.data_ptr(), bias.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+    check(rt_qkv_bias_split(input_data.data_ptr(), bias.data_ptr(), attention_q_from_rows() ? nullptr : q.data_ptr(),
+                            k.data_ptr(), v.data_ptr(),
                             seq_len_info_tensor.data_ptr<int>(), batch_size, block_num, head_num, scale,
                             dtype_code(input_data), current_stream()), "rt_qkv_bias_split");
     return;
@@ -239,7 +244,8 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
                       int batch_size, const torch::Tensor& seq_len_info_tensor, const torch::Tensor& from_select_index,
                       const torch::Tensor& from_select_index_position, const int* to_select_index,
                       const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
-                      int head_num, std::map<std::string, float>& info, bool balanced, const torch::Tensor& seq_tokens) {
+                      int head_num, std::map<std::string, float>& info, bool balanced, const torch::Tensor& seq_tokens,
+                      const torch::Tensor& qkv_rows, const torch::Tensor& qkv_bias) {
   ScopedGpuTimer timer(info, "attention");
   const int* tokens = nullptr;
   if (seq_tokens.defined() && seq_tokens.numel() > 0) {
@@ -259,6 +265,19 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
     from_idx = from_select_index.data_ptr<int>();
     from_pos = from_select_index_position.data_ptr<int>();
     n_wg = block_limit;
+  }
+  if (qkv_rows.defined()) {
+    require_cuda_contiguous(qkv_rows, "qkv_rows");
+    require_cuda_contiguous(qkv_bias, "qkv_bias");
+    if (qkv_rows.dim() != 2 || qkv_rows.size(0) != int64_t(block_num) * 64 || qkv_rows.size(1) != int64_t(head_num) * 192 ||
+        qkv_bias.numel() != qkv_rows.size(1) || qkv_rows.scalar_type() != out.scalar_type() ||
+        qkv_bias.scalar_type() != out.scalar_type())
+      throw std::invalid_argument("sparse_attention: qkv_rows must be [tokens, 3 * heads * 64] with a bias of that width");
+    check(rt_bs_attention_fwd_qrows(qkv_rows.data_ptr(), qkv_bias.data_ptr(), kQScale, k.data_ptr(), v.data_ptr(),
+                                    out.data_ptr(), seq_len_info_tensor.data_ptr<int>(), tokens, batch_size, block_num,
+                                    head_num, to_select_index, to_select_index_position, plan_heads, from_idx, from_pos,
+                                    n_wg, dtype_code(out), current_stream()), "rt_bs_attention_fwd_qrows");
+    return;
   }
   check(rt_bs_attention_fwd_masked(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                    seq_len_info_tensor.data_ptr<int>(), tokens, batch_size, block_num, head_num,

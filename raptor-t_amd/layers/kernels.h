@@ -68,6 +68,12 @@ void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch:
 void set_gemm_epilogue_fusion(bool on);
 bool gemm_epilogue_fusion();
 
+// Whether, under kernel_fusion, the attention kernel takes its queries from the QKV projection's
+// own output rows (bias and scale applied as each unit loads its tile) and the split kernel writes
+// only K and V^T (default), or the split kernel materialises Q too, as the reference always does.
+void set_attention_q_from_rows(bool on);
+bool attention_q_from_rows();
+
 // layers/kernels/add_bias_and_transpose.cu:212-233
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,
                                    torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,
@@ -90,9 +96,12 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
                       const torch::Tensor& from_select_index_position, const int* to_select_index,
                       const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
                       int head_num, std::map<std::string, float>& info, bool balanced,
-                      const torch::Tensor& seq_tokens = torch::Tensor());
+                      const torch::Tensor& seq_tokens = torch::Tensor(), const torch::Tensor& qkv_rows = torch::Tensor(),
+                      const torch::Tensor& qkv_bias = torch::Tensor());
 // seq_tokens (optional, int32 on the GPU, one entry per sequence): true token counts of sequences
 // whose last block ends in padding; the padded keys get no weight.
+// qkv_rows + qkv_bias (optional, the [T, 3*H*64] projection output and its bias): the queries are
+// read from there and `q` is ignored.
 
 }  // namespace kernels
 }  // namespace layers

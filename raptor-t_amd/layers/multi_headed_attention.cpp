@@ -101,9 +101,13 @@ void MultiHeadedAttention::operator()(const torch::Tensor& input_tensor, const t
   if (pre != info.end()) pre->second += float(wait_us);
 
   torch::Tensor attention_out = tensor_set->get_tensor("attention_out");
+  // under kernel_fusion the split kernel may have left Q in the projection's output (see kernels.h)
+  const bool q_rows = kernel_fusion && kernels::attention_q_from_rows();
   kernels::sparse_attention(q_out, k_out, v_out, attention_out, batch_size_, seq_len_info_tensor,
                             from_select_index_tensor, from_select_index_position_tensor, to_idx, to_pos, plan_heads,
-                            block_limit, block_num_, head_num_, info, balanced, attention_mask);
+                            block_limit, block_num_, head_num_, info, balanced, attention_mask,
+                            q_rows ? tensor_set->get_tensor("tmp_qkv_out1") : torch::Tensor(),
+                            q_rows ? qkv_bias_ : torch::Tensor());
   semaphore->Release(layer_idx_, stream);
 
   kernels::MatMul(attention_out, false, dense_weight_, true, 1, output, 0, handle_, "Attention Output");

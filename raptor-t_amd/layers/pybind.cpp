@@ -21,6 +21,11 @@ PYBIND11_MODULE(raptor_t, m) {
         "BertIntermediate with kernel_fusion runs bias + GELU in the GEMM's epilogue (True, the default) or as the "
         "separate add_bias_act kernel (False).");
   m.def("gemm_epilogue_fusion", &layers::kernels::gemm_epilogue_fusion);
+  m.def("set_attention_q_from_rows", &layers::kernels::set_attention_q_from_rows,
+        "With kernel_fusion the attention kernel reads its queries from the QKV projection's output and the split "
+        "kernel writes only K and V (True, the default), or the split kernel also writes Q (False).  Set it "
+        "between layer calls, not during one.");
+  m.def("attention_q_from_rows", &layers::kernels::attention_q_from_rows);
   m.def("timing_collect", &layers::kernels::timing_collect,
         "Synchronise and return {launcher: (total microseconds, launches)} since timing_begin().");
   py::class_<layers::BertAttention>(m, "BertAttention")

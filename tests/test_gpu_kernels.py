@@ -115,6 +115,45 @@ def test_attention_rows_longer_than_64_blocks(capi, n_wg):
     assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("dtype,n_wg,padded", [(torch.float16, 0, False), (torch.bfloat16, 0, False),
+                                               (torch.float16, 96, False), (torch.float16, 0, True)])
+def test_attention_queries_from_projection_rows(capi, dtype, n_wg, padded):
+    """rt_bs_attention_fwd_qrows (queries read from the [T, 3*H*64] projection output, bias and scale applied on
+    load; the split kernel called without a Q output) gives the same bits as the route through a materialised Q,
+    and both match the oracle."""
+    say("attention qrows", dtype, n_wg, padded)
+    heads, seq_lens = 4, [64 * 13, 64 * 3, 64 * 20, 64]
+    t, dm = sum(seq_lens), heads * 64
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(t, 3 * dm, generator=g).to(dtype).cuda()
+    bias = (torch.randn(3 * dm, generator=g) * 0.5).to(dtype).cuda()
+    sb, idx, pos, ph, sb_d, idx_d, pos_d = lh.device_plan(capi, seq_lens, heads, 0, None)
+    seq_tokens = [n - 17 for n in seq_lens] if padded else None
+    tok_d = None if seq_tokens is None else torch.tensor(seq_tokens, dtype=torch.int32).cuda()
+    from_idx = from_pos = None
+    if n_wg:
+        fp, fi = capi.partition_lpt(sb, heads, n_wg)
+        from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
+    new = lambda: torch.full((t * dm,), float("nan"), dtype=dtype, device="cuda")
+    q, k, vt, k2, vt2 = new(), new(), new(), new(), new()
+    out_a, out_b = new().view(t, dm), new().view(t, dm)
+    capi.qkv_bias_split(qkv, bias, q, k, vt, sb_d, heads, capi.Q_SCALE)
+    capi.bs_attention_fwd(q, k, vt, out_a, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos, tok_d)
+    capi.qkv_bias_split(qkv, bias, None, k2, vt2, sb_d, heads, capi.Q_SCALE)
+    capi.bs_attention_fwd_qrows(qkv, bias, capi.Q_SCALE, k2, vt2, out_b, sb_d, heads, idx_d, pos_d, ph, from_idx,
+                                from_pos, tok_d)
+    torch.cuda.synchronize()
+    assert torch.equal(k, k2) and torch.equal(vt, vt2)
+    assert torch.equal(out_a, out_b)
+    x = qkv.float().cpu() + bias.float().cpu()
+    qs = (x[:, :dm] * capi.Q_SCALE).to(dtype).view(t, heads, 64)
+    kk, vv = (x[:, i * dm:(i + 1) * dm].to(dtype).view(t, heads, 64) for i in (1, 2))
+    ref = oa.csr_attention(qs, kk, vv, sb.tolist(), idx, pos, ph, scale=1.0 / lh.LOG2E, seq_tokens=seq_tokens)
+    assert (out_b.float().cpu() - ref).abs().max().item() <= 2e-2
+    with pytest.raises(capi.RaptorError):
+        capi.bs_attention_fwd_qrows(qkv, None, capi.Q_SCALE, k2, vt2, out_b, sb_d, heads, idx_d, pos_d, ph)
+
+
 def test_attention_maximum_batch(capi):
     """1024 sequences in one launch is the limit of the kernel's LDS geometry tables; one more is refused."""
     say("attention max batch")

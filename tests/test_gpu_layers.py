@@ -108,6 +108,13 @@ def test_fused_and_unfused_paths_agree(mb, ut):
         assert ("add_bias_act_kernel" in ran) == (not (fused and epilogue))
         outs.append(out.float().cpu())
     mb.cxx.set_gemm_epilogue_fusion(True)
+    # queries read from the projection's rows (default) / materialised by the split kernel: same bits
+    assert mb.cxx.attention_q_from_rows()
+    mb.cxx.set_attention_q_from_rows(False)
+    meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+    out, _ = layer(x.clone(), spi, spi_t, ppi_t, pp_t, new(ffn), new(hidden), new(hidden), 64, kernel_fusion=True)
+    mb.cxx.set_attention_q_from_rows(True)
+    assert torch.equal(out.float().cpu(), outs[0])
     meta.terminate_thread()
     assert (outs[0] - outs[1]).abs().max().item() <= 2e-2
     assert (outs[0] - outs[2]).abs().max().item() <= 2e-2
