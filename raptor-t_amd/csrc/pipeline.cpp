@@ -255,7 +255,13 @@ int rt_pipeline_acquire(rt_pipeline* p, int layer, void* stream, const int** to_
   }
   Slot& s = L.slot[gen & 1];
   if (p->device >= 0) {
-    HIP_TRY(hipStreamWaitEvent((hipStream_t)stream, s.copied, 0));
+    // The workers run ahead of the layers: the upload has usually finished long before its layer is
+    // reached, and then the compute stream needs no barrier (one costs several microseconds of idle GPU).
+    const hipError_t done = hipEventQuery(s.copied);
+    if (done != hipSuccess) {
+      (void)hipGetLastError();                       // hipErrorNotReady is not a failure
+      HIP_TRY(hipStreamWaitEvent((hipStream_t)stream, s.copied, 0));
+    }
     *to_idx = s.dev_idx;
     *to_pos = s.dev_pos;
   } else {
