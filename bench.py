@@ -285,6 +285,12 @@ def run_streaming(args):
         enc(h, t, args.block_limit, spi, spi_t, ppi_t, pp_t, tmp[:t], inter[:t], attn[:t], test_info={},
             balanced=args.lpt_plan)
 
+    # Start-up tuning, as a server does once: the GEMMs of every token count the batches can have (16 sequences of
+    # 512..4096 tokens in steps of 64).  Without it the first batch of each token count stalls ~17 ms on timing
+    # six candidate kernels per GEMM; --no-pretune shows that.
+    tune_s = 0.0
+    if not args.no_pretune:
+        tune_s = mb.cxx.tune_layer_gemms(list(range(16 * 512, 16 * 4096 + 1, 64)), hidden, ffn, dt)
     for b in batches[:args.warmup]:
         step(b)
     torch.cuda.synchronize()
@@ -301,7 +307,8 @@ def run_streaming(args):
             "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "stream: config 3's encoder, a new batch of 16 lengths U[512,4096] every step",
                        "balanced": args.lpt_plan, "block_limit": args.block_limit},
-            "tokens_per_s": tokens / elapsed, "host_batch_metadata_ms_per_step": host_prep[0] / args.steps * 1e3}
+            "tokens_per_s": tokens / elapsed, "host_batch_metadata_ms_per_step": host_prep[0] / args.steps * 1e3,
+            "gemm_startup_tuning_s": tune_s}
 
 
 def main():
@@ -319,6 +326,8 @@ def main():
     ap.add_argument("--materialize-q", action="store_true",
                     help="the split kernel writes Q too and the attention kernel reads it from there (the reference's "
                          "arrangement) instead of taking its queries from the projection's output rows")
+    ap.add_argument("--no-pretune", action="store_true",
+                    help="stream workload: skip the start-up GEMM tuning over the range of token counts")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=2)
     args = ap.parse_args()

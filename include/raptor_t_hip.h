@@ -199,6 +199,11 @@ int rt_gemm_destroy(rt_gemm_ctx* ctx);
  * the problem (seconds per kind, once per process). */
 #define RT_GEMM_TUNE_ALL (-1)
 int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates);
+/* A packed batch brings a new M with every batch, and the fastest solution moves with M (output
+ * tiles against CUs).  The first call with a new M of a kind already tuned times only that
+ * kind's `candidates` best solutions (default 6, about 3 ms; at most 8); 0 or 1 = take the
+ * kind's winner untimed.  A server that knows its range of token counts runs each once at start. */
+int rt_gemm_set_retuning(rt_gemm_ctx* ctx, int candidates);
 int rt_gemm(rt_gemm_ctx* ctx, const void* a, const void* b, void* c,
             int64_t m, int64_t n, int64_t k, int dtype, void* stream);
 

@@ -24,7 +24,7 @@ EXPORTS = [
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows",
-    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm",
+    "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm_set_retuning", "rt_gemm",
     "rt_gemm_bias_act", "rt_gemm_bt",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
@@ -67,6 +67,7 @@ def lib():
         L.rt_gemm_create.argtypes = [ctypes.POINTER(vp)]
         L.rt_gemm_destroy.argtypes = [vp]
         L.rt_gemm_set_tuning.argtypes = [vp, I]
+        L.rt_gemm_set_retuning.argtypes = [vp, I]
         L.rt_gemm.argtypes = [vp, vp, vp, vp, L64, L64, L64, I, vp]
         L.rt_embed_layernorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, L64, I, I, I, I, ctypes.c_float, I, I, vp]
         L.rt_gemm_bias_act.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
@@ -257,6 +258,10 @@ class Gemm:
 
     def set_tuning(self, candidates):
         check(lib().rt_gemm_set_tuning(self._h, candidates))
+
+    def set_retuning(self, candidates):
+        """How many of a kind's best solutions the first call with a new M times (0 / 1: none)."""
+        check(lib().rt_gemm_set_retuning(self._h, candidates))
 
     def __call__(self, a, b, c):
         m, k = a.shape

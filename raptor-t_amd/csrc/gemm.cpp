@@ -18,6 +18,7 @@
 #include <hipblaslt/hipblaslt.h>
 #include <hipblaslt/hipblaslt-ext.hpp>
 
+#include <algorithm>
 #include <map>
 #include <vector>
 #include <mutex>
@@ -40,9 +41,11 @@ struct rt_gemm_ctx {
   };
   // keyed by (M, N, K, dtype, mode); mode = epilogue | MODE_B_TRANS
   std::map<std::tuple<int64_t, int64_t, int64_t, int, int>, Plan> plans;
-  // winning solution index per (N, K, dtype, mode): a packed batch changes M with every
-  // batch, the timing run is not repeated for each new M
-  std::map<std::tuple<int64_t, int64_t, int, int>, int> tuned_index;
+  // The fastest solutions (library indices, best first) of the first M seen of each (N, K, dtype,
+  // mode).  A packed batch changes M with every batch and the best solution moves with it (the
+  // number of output tiles against the number of CUs), so each further M times only these.
+  std::map<std::tuple<int64_t, int64_t, int, int>, std::vector<int>> kind_best;
+  int retune_candidates = 6;        // how many of kind_best a further M times (<= 1: take the first untimed)
 };
 
 namespace {
@@ -99,22 +102,41 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int 
     LT_TRY(hipblasLtMatrixLayoutCreate(&p.la, t, n, k, n));
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.lb, t, k, m, k));
   LT_TRY(hipblasLtMatrixLayoutCreate(&p.lc, t, n, m, n));
-  // A packed batch changes M with every batch.  Once a (N, K, dtype, mode) has a winner, a new M
-  // takes it by its index, without asking the heuristic again (cheaper on the host, and the winner of
-  // an exhaustive search need not be among the heuristic's suggestions).
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  const bool can_time = hipStreamIsCapturing(st, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone;
+  // A further M of a known kind: time the kind's best few (not the whole candidate list again).
   {
-    auto known = ctx->tuned_index.find(std::make_tuple(n, k, dtype, mode));
-    if (known != ctx->tuned_index.end()) {
-      std::vector<int> index{known->second};
+    auto known = ctx->kind_best.find(std::make_tuple(n, k, dtype, mode));
+    if (known != ctx->kind_best.end() && !known->second.empty()) {
+      const int want = ctx->retune_candidates < 1 ? 1 : ctx->retune_candidates;
+      std::vector<int> index(known->second.begin(),
+                             known->second.begin() + std::min<size_t>(known->second.size(), size_t(want)));
       std::vector<hipblasLtMatmulHeuristicResult_t> byindex;
       const float one = 1.0f, zero = 0.0f;
-      size_t ws = 0;
-      if (hipblaslt_ext::getAlgosFromIndex(ctx->lt, index, byindex) == HIPBLAS_STATUS_SUCCESS && !byindex.empty() &&
-          hipblaslt_ext::matmulIsAlgoSupported(ctx->lt, p.desc, &one, p.la, p.lb, &zero, p.lc, p.lc, byindex[0].algo, ws) ==
-              HIPBLAS_STATUS_SUCCESS && ws <= ctx->workspace_bytes) {
-        p.algo = byindex[0].algo;
-        p.ws = ws;
-        return RT_OK;
+      if (hipblaslt_ext::getAlgosFromIndex(ctx->lt, index, byindex) == HIPBLAS_STATUS_SUCCESS) {
+        std::vector<std::pair<hipblasLtMatmulAlgo_t, size_t>> ok;
+        for (auto& r : byindex) {
+          size_t ws = 0;
+          if (hipblaslt_ext::matmulIsAlgoSupported(ctx->lt, p.desc, &one, p.la, p.lb, &zero, p.lc, p.lc, r.algo, ws) ==
+                  HIPBLAS_STATUS_SUCCESS && ws <= ctx->workspace_bytes)
+            ok.emplace_back(r.algo, ws);
+        }
+        if (!ok.empty()) {
+          size_t best = 0;
+          hipEvent_t e0 = nullptr, e1 = nullptr;
+          if (ok.size() > 1 && can_time && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+            float best_ms = -1.f;
+            for (size_t i = 0; i < ok.size(); ++i) {
+              const float ms = time_algo(ctx, p, ok[i].first, a, b, c, st, e0, e1);
+              if (ms > 0.f && (best_ms < 0.f || ms < best_ms)) { best_ms = ms; best = i; }
+            }
+          }
+          if (e0) (void)hipEventDestroy(e0);
+          if (e1) (void)hipEventDestroy(e1);
+          p.algo = ok[best].first;
+          p.ws = ok[best].second;
+          return RT_OK;
+        }
       }
     }
   }
@@ -133,7 +155,7 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int 
     return rt::fail(RT_ENOSYS, "hipBLASLt has no algorithm for M=%lld N=%lld K=%lld dtype=%d (status %d)", (long long)m,
                     (long long)n, (long long)k, dtype, int(hs));
   res.resize(found);
-  if (ctx->tune_candidates == RT_GEMM_TUNE_ALL && !ctx->tuned_index.count(std::make_tuple(n, k, dtype, mode))) {
+  if (ctx->tune_candidates == RT_GEMM_TUNE_ALL) {
     // every solution the library has for these types, filtered to the ones that accept this problem
     std::vector<hipblasLtMatmulHeuristicResult_t> all;
     if (hipblaslt_ext::getAllAlgos(ctx->lt, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, first_op, HIPBLAS_OP_N, t, t, t, t,
@@ -151,36 +173,37 @@ int make_plan(rt_gemm_ctx* ctx, int64_t m, int64_t n, int64_t k, int dtype, int 
       found = int(res.size());
     }
   }
-  int best = -1;
-  auto tuned = ctx->tuned_index.find(std::make_tuple(n, k, dtype, mode));
-  if (tuned != ctx->tuned_index.end())
-    for (int i = 0; i < found && best < 0; ++i)
-      if (res[i].state == HIPBLAS_STATUS_SUCCESS && hipblaslt_ext::getIndexFromAlgo(res[i].algo) == tuned->second) best = i;
-  if (best >= 0) {
-    p.algo = res[best].algo;
-    p.ws = res[best].workspaceSize;
-    return RT_OK;
-  }
-  best = 0;
   // The library's first suggestion is often not the fastest for these tall, K=768 shapes: time the
-  // candidates once per shape on the caller's own operands (skipped while a graph is being captured).
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (found > 1 && hipStreamIsCapturing(st, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone) {
+  // candidates once per kind on the caller's own operands (skipped while a graph is being captured),
+  // then the best eight a second time (the ranking of near-equal candidates is noisy) and keep their order.
+  std::vector<std::pair<float, int>> ranked;          // (milliseconds, position in res)
+  if (found > 1 && can_time) {
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
-      float best_ms = -1.f;
       for (int i = 0; i < found; ++i) {
         if (res[i].state != HIPBLAS_STATUS_SUCCESS || res[i].workspaceSize > ctx->workspace_bytes) continue;
         const float ms = time_algo(ctx, p, res[i].algo, a, b, c, st, e0, e1);
-        if (ms > 0.f && (best_ms < 0.f || ms < best_ms)) { best_ms = ms; best = i; }
+        if (ms > 0.f) ranked.emplace_back(ms, i);
       }
+      std::sort(ranked.begin(), ranked.end());
+      if (ranked.size() > 8) ranked.resize(8);
+      for (auto& r : ranked) {
+        const float ms = time_algo(ctx, p, res[r.second].algo, a, b, c, st, e0, e1);
+        if (ms > 0.f && ms < r.first) r.first = ms;
+      }
+      std::sort(ranked.begin(), ranked.end());
     }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
   }
+  const int best = ranked.empty() ? 0 : ranked[0].second;
   p.algo = res[best].algo;
   p.ws = res[best].workspaceSize;
-  ctx->tuned_index[std::make_tuple(n, k, dtype, mode)] = hipblaslt_ext::getIndexFromAlgo(res[best].algo);
+  if (!ranked.empty()) {
+    std::vector<int> order;
+    for (auto& r : ranked) order.push_back(hipblaslt_ext::getIndexFromAlgo(res[r.second].algo));
+    ctx->kind_best[std::make_tuple(n, k, dtype, mode)] = order;
+  }
   return RT_OK;
 }
 
@@ -227,6 +250,14 @@ int rt_gemm_set_tuning(rt_gemm_ctx* ctx, int candidates) {
              "candidates=%d must be in [1, 64] or RT_GEMM_TUNE_ALL", candidates);
   std::lock_guard<std::mutex> lk(ctx->m);
   ctx->tune_candidates = candidates;
+  return RT_OK;
+}
+
+int rt_gemm_set_retuning(rt_gemm_ctx* ctx, int candidates) {
+  RT_REQUIRE(ctx, RT_EINVAL, "NULL context");
+  RT_REQUIRE(candidates >= 0 && candidates <= 8, RT_EINVAL, "candidates=%d must be in [0, 8]", candidates);
+  std::lock_guard<std::mutex> lk(ctx->m);
+  ctx->retune_candidates = candidates;
   return RT_OK;
 }
 

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <atomic>
+#include <chrono>
 #include <cmath>
 #include <mutex>
 #include <set>
@@ -164,6 +165,34 @@ void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch:
   else
     check(rt_gemm_bias_act(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), n, A.size(1),
                            RT_EPILOGUE_BIAS_GELU, dtype_code(A), current_stream()), name.c_str());
+}
+
+double tune_layer_gemms(const std::vector<int64_t>& token_counts, int64_t hidden, int64_t ffn, torch::ScalarType dtype) {
+  if (token_counts.empty()) return 0.0;
+  if (hidden <= 0 || ffn <= 0) throw std::invalid_argument("tune_layer_gemms: hidden and ffn must be positive");
+  int64_t max_m = 0;
+  for (int64_t m : token_counts) {
+    if (m <= 0) throw std::invalid_argument("tune_layer_gemms: token counts must be positive");
+    max_m = std::max(max_m, m);
+  }
+  const auto t0 = std::chrono::steady_clock::now();
+  auto opt = torch::TensorOptions().dtype(dtype).device(torch::kCUDA);
+  const int64_t wide = std::max(3 * hidden, ffn);
+  // random operands: an all-zero product draws less power and would be timed at other clocks
+  torch::Tensor a = torch::randn({max_m, wide}, opt), out = torch::empty({max_m, wide}, opt);
+  torch::Tensor w = torch::randn({wide, wide}, opt) * 0.05, bias = torch::zeros({wide}, opt);
+  rt_gemm_ctx* handle = shared_gemm_handle();
+  void* stream = current_stream();
+  const int dt = dtype_code(a);
+  for (int64_t m : token_counts) {
+    const int64_t shapes[4][3] = {{3 * hidden, hidden, RT_EPILOGUE_NONE}, {hidden, hidden, RT_EPILOGUE_NONE},
+                                  {ffn, hidden, RT_EPILOGUE_BIAS_GELU}, {hidden, ffn, RT_EPILOGUE_NONE}};
+    for (const auto& sh : shapes)
+      check(rt_gemm_bt(handle, a.data_ptr(), w.data_ptr(), sh[2] == RT_EPILOGUE_NONE ? nullptr : bias.data_ptr(),
+                       out.data_ptr(), m, sh[0], sh[1], int(sh[2]), dt, stream), "tune_layer_gemms");
+  }
+  check(hipStreamSynchronize(static_cast<hipStream_t>(stream)) == hipSuccess ? 0 : RT_EIO, "tune_layer_gemms");
+  return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
 }
 
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,

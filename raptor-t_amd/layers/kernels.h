@@ -74,6 +74,12 @@ bool gemm_epilogue_fusion();
 void set_attention_q_from_rows(bool on);
 bool attention_q_from_rows();
 
+// Start-up tuning for a server: runs the four GEMMs of an encoder layer (hidden -> 3*hidden,
+// hidden -> hidden, hidden -> ffn with bias + GELU, ffn -> hidden; weights as [out, in]) once for every
+// token count in `token_counts` on the shared context, so that no later batch of one of these sizes
+// pays for the timing of candidates.  Uses scratch operands of its own; returns the seconds it took.
+double tune_layer_gemms(const std::vector<int64_t>& token_counts, int64_t hidden, int64_t ffn, torch::ScalarType dtype);
+
 // layers/kernels/add_bias_and_transpose.cu:212-233
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,
                                    torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,

@@ -21,6 +21,14 @@ PYBIND11_MODULE(raptor_t, m) {
         "BertIntermediate with kernel_fusion runs bias + GELU in the GEMM's epilogue (True, the default) or as the "
         "separate add_bias_act kernel (False).");
   m.def("gemm_epilogue_fusion", &layers::kernels::gemm_epilogue_fusion);
+  m.def("tune_layer_gemms",
+        [](const std::vector<int64_t>& token_counts, int64_t hidden, int64_t ffn, py::object dtype) {
+          return layers::kernels::tune_layer_gemms(token_counts, hidden, ffn,
+                                                   torch::python::detail::py_object_to_dtype(dtype));
+        },
+        py::arg("token_counts"), py::arg("hidden"), py::arg("ffn"), py::arg("dtype"),
+        "Run the four GEMMs of an encoder layer once for every token count (start-up tuning of a server: the first "
+        "call with a new token count times a few candidate kernels); returns the seconds spent.");
   m.def("set_attention_q_from_rows", &layers::kernels::set_attention_q_from_rows,
         "With kernel_fusion the attention kernel reads its queries from the QKV projection's output and the split "
         "kernel writes only K and V (True, the default), or the split kernel also writes Q (False).  Set it "

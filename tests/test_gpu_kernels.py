@@ -300,6 +300,28 @@ def test_gemm_exhaustive_tuning_keeps_results(capi):
     gemm = capi.Gemm()
     with pytest.raises(capi.RaptorError):
         gemm.set_tuning(0)
+    with pytest.raises(capi.RaptorError):
+        gemm.set_retuning(9)
+    gemm.close()
+
+
+@pytest.mark.parametrize("retune", [0, 3, 8])
+def test_gemm_retuning_for_new_token_counts_keeps_results(capi, retune):
+    """A new M of a kind already tuned times `retune` of the kind's best solutions (or none): same results."""
+    say("gemm retune", retune)
+    g = torch.Generator().manual_seed(6)
+    a = torch.randn(1000, 256, generator=g).half().cuda()
+    bt = (torch.randn(384, 256, generator=g) * 0.05).half().cuda()
+    bias = torch.randn(384, generator=g).half().cuda()
+    want = ol.bias_gelu(a.double().cpu() @ bt.double().cpu().t(), bias.cpu())
+    gemm = capi.Gemm()
+    gemm.set_retuning(retune)
+    for rows in (1000, 640, 64, 1):
+        c = torch.empty(rows, 384, dtype=torch.float16, device="cuda")
+        for _ in range(2):                                  # the second call takes the cached plan
+            gemm.bt(a[:rows].contiguous(), bt, c, bias=bias, epilogue=capi.RT_EPILOGUE_BIAS_GELU)
+            torch.cuda.synchronize()
+            assert (c.double().cpu() - want[:rows]).abs().max().item() <= 2e-2
     gemm.close()
 
 

@@ -120,6 +120,15 @@ def test_fused_and_unfused_paths_agree(mb, ut):
     assert (outs[0] - outs[2]).abs().max().item() <= 2e-2
 
 
+def test_startup_gemm_tuning_runs(mb):
+    say("tune_layer_gemms")
+    assert mb.cxx.tune_layer_gemms([], 768, 3072, torch.float16) == 0.0
+    assert mb.cxx.tune_layer_gemms([128, 192, 64], 256, 512, torch.float16) > 0.0
+    assert mb.cxx.tune_layer_gemms([128], 256, 512, torch.bfloat16) > 0.0
+    with pytest.raises(Exception):
+        mb.cxx.tune_layer_gemms([0], 256, 512, torch.float16)
+
+
 def test_api_rejects_mismatched_batch(mb, ut):
     hidden, heads, ffn, dtype = 768, 12, 3072, torch.float16
     g = torch.Generator().manual_seed(2)
