@@ -417,13 +417,15 @@ template <typename T> __device__ inline void store8(T* p, const float* x) {
   for (int i = 0; i < 8; i += N) Vec<T>::store(p + i, x + i);
 }
 
-template <typename T>
+template <typename T, bool WITH_Q>
 __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict__ qkv, const T* __restrict__ bias,
                                                              T* __restrict__ q, T* __restrict__ k,
                                                              T* __restrict__ vt, const int* __restrict__ seq_blocks,
                                                              int batch, int heads, float q_scale) {
   constexpr int N = Vec<T>::N;              // elements per 16 bytes
   constexpr int CPR = 64 / N;               // 16-byte chunks per 64-wide row
+  constexpr int ITERS = 64 * CPR / 256;     // chunks per thread and matrix
+  constexpr int M0 = WITH_Q ? 0 : 1;        // without Q (left to the attention kernel) only K and V are read
   // Only V needs a transpose.  A Q / K fragment entry (8 consecutive d of one token) is a run of the
   // source row already: those two matrices are copied run by run to their permuted places.
   __shared__ float vtile[64][65];
@@ -432,18 +434,27 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
   // power-of-two head count, one XCD (workgroups go to the 8 XCDs round-robin) does not always get
   // the same heads' columns.
   const int g = blockIdx.x / heads, h = (blockIdx.x % heads + g) % heads;
+  const int dm = heads * 64;
+  const T* src = qkv + int64_t(g) * 64 * (3 * dm) + h * 64;
+  // every load of the thread is issued before anything waits for one: the kernel lives on bytes in flight
+  uint4 raw[ITERS][3];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = threadIdx.x + it * 256, row = c / CPR, col = (c % CPR) * N;
+#pragma unroll
+    for (int m = M0; m < 3; ++m)
+      raw[it][m] = *reinterpret_cast<const uint4*>(src + int64_t(row) * 3 * dm + m * dm + col);
+  }
   const int s = find_seq(seq_blocks, batch, g);
   const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
   const int64_t base = (int64_t(g0) * heads + int64_t(h) * n + (g - g0)) * 4096;
-  const int dm = heads * 64;
-  const T* src = qkv + int64_t(g) * 64 * (3 * dm) + h * 64;
-  for (int c = threadIdx.x; c < 64 * CPR; c += 256) {
-    const int row = c / CPR, col = (c % CPR) * N;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = threadIdx.x + it * 256, row = c / CPR, col = (c % CPR) * N;
     float x[3][N], b[3][N];
 #pragma unroll
-    for (int m = 0; m < 3; ++m) {
-      if (m == 0 && !q) continue;                       // Q is left to the attention kernel
-      Vec<T>::load(src + int64_t(row) * 3 * dm + m * dm + col, x[m]);
+    for (int m = M0; m < 3; ++m) {
+      Vec<T>::load(reinterpret_cast<const T*>(&raw[it][m]), x[m]);
       Vec<T>::load(bias + m * dm + h * 64 + col, b[m]);
     }
     // run `col8` (8 elements) of token `row` is lane (row & 31) + 32 * (col8 & 1) of fragment
@@ -452,15 +463,17 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
     const int dst = ((4 * (row >> 5) + (col8 >> 1)) * 64 + (row & 31) + 32 * (col8 & 1)) * 8 + (col & 7);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      if (q) x[0][i] = (x[0][i] + b[0][i]) * q_scale;
+      if (WITH_Q) x[0][i] = (x[0][i] + b[0][i]) * q_scale;
       x[1][i] = x[1][i] + b[1][i];
       vtile[row][col + i] = x[2][i] + b[2][i];
     }
-    if (q) Vec<T>::store(q + base + dst, x[0]);
+    if (WITH_Q) Vec<T>::store(q + base + dst, x[0]);
     Vec<T>::store(k + base + dst, x[1]);
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < 512; c += 256) {
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    const int c = threadIdx.x + it * 256;
     const int f = c >> 6, l = c & 63;
     const int r32 = 32 * (f >> 2) + (l & 31), c8 = 16 * (f & 3) + 8 * (l >> 5);
     float x[8];
@@ -556,16 +569,18 @@ int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void*
              "pointers must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid(unsigned(heads) * unsigned(total_blocks));
-  if (dtype == RT_F16)
-    hipLaunchKernelGGL(qkv_bias_split_kernel<__half>, grid, dim3(256), 0, st, (const __half*)qkv, (const __half*)bias,
-                       (__half*)q, (__half*)k, (__half*)vt, seq_blocks_dev, batch, heads, q_scale);
-  else if (dtype == RT_BF16)
-    hipLaunchKernelGGL(qkv_bias_split_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)qkv,
-                       (const __hip_bfloat16*)bias, (__hip_bfloat16*)q, (__hip_bfloat16*)k, (__hip_bfloat16*)vt,
-                       seq_blocks_dev, batch, heads, q_scale);
-  else
-    hipLaunchKernelGGL(qkv_bias_split_kernel<float>, grid, dim3(256), 0, st, (const float*)qkv, (const float*)bias,
-                       (float*)q, (float*)k, (float*)vt, seq_blocks_dev, batch, heads, q_scale);
+  auto launch = [&](auto tag) {
+    typedef decltype(tag) T;
+    if (q)
+      hipLaunchKernelGGL((qkv_bias_split_kernel<T, true>), grid, dim3(256), 0, st, (const T*)qkv, (const T*)bias, (T*)q,
+                         (T*)k, (T*)vt, seq_blocks_dev, batch, heads, q_scale);
+    else
+      hipLaunchKernelGGL((qkv_bias_split_kernel<T, false>), grid, dim3(256), 0, st, (const T*)qkv, (const T*)bias,
+                         (T*)nullptr, (T*)k, (T*)vt, seq_blocks_dev, batch, heads, q_scale);
+  };
+  if (dtype == RT_F16) launch(__half());
+  else if (dtype == RT_BF16) launch(__hip_bfloat16());
+  else launch(float());
   return check_launch("qkv_bias_split");
 }
 
