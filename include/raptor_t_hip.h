@@ -224,6 +224,21 @@ int rt_gemm_bias_act(rt_gemm_ctx* ctx, const void* a, const void* b, const void*
 int rt_gemm_bt(rt_gemm_ctx* ctx, const void* a, const void* bt, const void* bias, void* c,
                int64_t m, int64_t n, int64_t k, int epilogue, int dtype, void* stream);
 
+/* ------------------------------------------------------------------ pooling + pooler head */
+
+/* SequencePool of the reference (python/modeling_bert.py:270-277, a stub there; the modes are its
+ * PoolingType, :298-314) for a packed batch: out[s, :] = the first / last token's row of sequence
+ * s, or the mean / maximum over its tokens (fp32 accumulation).  seq_tokens_dev (optional) gives
+ * the true token counts of sequences whose last block ends in padding. */
+enum { RT_POOL_FIRST = 0, RT_POOL_LAST = 1, RT_POOL_MEAN = 2, RT_POOL_MAX = 3 };
+int rt_sequence_pool(const void* hidden, const int* seq_blocks_dev, const int* seq_tokens_dev,
+                     int batch, int width, int mode, void* out, int dtype, void* stream);
+
+/* BertPooler (python/modeling_bert.py:279-296, commented out in the reference; HuggingFace
+ * BigBirdModel.pooler + tanh): out[B, d_out] = tanh(pooled[B, d_in] . weight_t[d_out, d_in]^T + bias). */
+int rt_pooler_dense_tanh(const void* pooled, const void* weight_t, const void* bias, void* out,
+                         int batch, int d_in, int d_out, int dtype, void* stream);
+
 /* ------------------------------------------------------- metadata / stream pipeline */
 
 /* Replaces Semaphore + MetaData + the per-layer std::async index workers

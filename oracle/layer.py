@@ -90,3 +90,35 @@ def random_layer_weights(hidden, ffn, generator, std=0.02, dtype=torch.float32):
         "out_weight": n(ffn, hidden), "out_bias": n(hidden),
         "out_ln_weight": torch.ones(hidden, dtype=dtype), "out_ln_bias": torch.zeros(hidden, dtype=dtype),
     }
+
+
+def sequence_pool(hidden, seq_blocks, mode, seq_tokens=None, block=64):
+    """SequencePool of the reference (python/modeling_bert.py:270-277 is a stub; modes = PoolingType,
+    :298-314) for a packed batch: per sequence the first / last token's row, or the mean / max over
+    its tokens.  hidden [T, D]; seq_tokens = true token counts when the last block ends in padding."""
+    hidden = hidden.double()
+    rows = []
+    for s in range(len(seq_blocks) - 1):
+        t0 = seq_blocks[s] * block
+        count = (seq_blocks[s + 1] - seq_blocks[s]) * block
+        if seq_tokens is not None:
+            count = max(1, min(int(seq_tokens[s]), count))
+        x = hidden[t0:t0 + count]
+        if mode == "First":
+            rows.append(x[0])
+        elif mode == "Last":
+            rows.append(x[-1])
+        elif mode == "Mean":
+            rows.append(x.sum(0) / count)
+        elif mode == "Max":
+            rows.append(x.max(0).values)
+        else:
+            raise ValueError("unknown pooling mode %r" % (mode,))
+    return torch.stack(rows).float()
+
+
+def pooler(pooled, weight, bias):
+    """BertPooler (python/modeling_bert.py:279-296, commented out there; HuggingFace
+    BigBirdModel: `activation(pooler(sequence_output[:, 0]))`, modeling_big_bird.py): tanh of a dense
+    layer; weight is [in, out] as every weight of the layers."""
+    return torch.tanh(pooled.double() @ weight.double() + bias.double()).float()

@@ -25,7 +25,7 @@ EXPORTS = [
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm_set_retuning", "rt_gemm",
-    "rt_gemm_bias_act", "rt_gemm_bt",
+    "rt_gemm_bias_act", "rt_gemm_bt", "rt_sequence_pool", "rt_pooler_dense_tanh",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
     "rt_pipeline_destroy",
 ]
@@ -72,6 +72,8 @@ def lib():
         L.rt_embed_layernorm.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, L64, I, I, I, I, ctypes.c_float, I, I, vp]
         L.rt_gemm_bias_act.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
         L.rt_gemm_bt.argtypes = [vp, vp, vp, vp, vp, L64, L64, L64, I, I, vp]
+        L.rt_sequence_pool.argtypes = [vp, vp, vp, I, I, I, vp, I, vp]
+        L.rt_pooler_dense_tanh.argtypes = [vp, vp, vp, vp, I, I, I, I, vp]
         L.rt_pipeline_create.argtypes = [ctypes.POINTER(vp), I, I, I, I, I, I, I]
         L.rt_pipeline_publish.argtypes = [vp, i32p, I]
         L.rt_pipeline_acquire.argtypes = [vp, I, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), i32p,
@@ -229,6 +231,32 @@ def bias_residual_layernorm(out, residual, bias, gamma, beta, eps):
 def bias_gelu(out, bias):
     rows, width = out.shape
     check(lib().rt_bias_gelu(_dp(out), _dp(bias), rows, width, _dtype_code(out), _stream()))
+
+
+RT_POOL_FIRST, RT_POOL_LAST, RT_POOL_MEAN, RT_POOL_MAX = 0, 1, 2, 3
+
+
+def sequence_pool(hidden, seq_blocks_dev, mode, out, seq_tokens_dev=None):
+    """out[s] = first / last token's row of sequence s, or the mean / max over its tokens (packed batch)."""
+    batch = seq_blocks_dev.numel() - 1
+    if tuple(out.shape) != (batch, hidden.shape[1]) or out.dtype != hidden.dtype:
+        raise ValueError("out must be [sequences, width] in the dtype of hidden")
+    if seq_tokens_dev is not None and seq_tokens_dev.numel() != batch:
+        raise ValueError("seq_tokens_dev needs one entry per sequence")
+    check(lib().rt_sequence_pool(_dp(hidden), _dp(seq_blocks_dev), _dp(seq_tokens_dev), batch, hidden.shape[1], mode,
+                                 _dp(out), _dtype_code(hidden), _stream()))
+    return out
+
+
+def pooler_dense_tanh(pooled, weight_t, bias, out):
+    """out = tanh(pooled @ weight_t.T + bias), weight_t as [out, in]."""
+    batch, d_in = pooled.shape
+    d_out = weight_t.shape[0]
+    if weight_t.shape[1] != d_in or bias.numel() != d_out or tuple(out.shape) != (batch, d_out):
+        raise ValueError("shape mismatch")
+    check(lib().rt_pooler_dense_tanh(_dp(pooled), _dp(weight_t), _dp(bias), _dp(out), batch, d_in, d_out,
+                                     _dtype_code(pooled), _stream()))
+    return out
 
 
 def embed_layernorm(input_ids, position_ids, token_type_ids, word, position, token_type, gamma, beta, out, eps=1e-12):

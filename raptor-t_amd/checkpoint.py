@@ -96,6 +96,16 @@ def convert_state_dict(sd):
     return emb, layers
 
 
+def pooler_from_state_dict(sd):
+    """-> (weight [in, out], bias) of the pooling head, or None when the checkpoint has none.
+    BigBird keeps it as `pooler.weight` (an nn.Linear), BERT as `pooler.dense.weight`."""
+    sd = _strip_prefix(sd)
+    for stem in ("pooler.", "pooler.dense."):
+        if stem + "weight" in sd and stem + "bias" in sd:
+            return torch.t(sd[stem + "weight"]).contiguous(), sd[stem + "bias"]
+    return None
+
+
 def load(path):
     """-> (embeddings, layers, config) of a local checkpoint; see convert_state_dict."""
     sd, cfg = read_state_dict(path)

@@ -503,6 +503,72 @@ __global__ __launch_bounds__(256) void unpack_head_tiles_kernel(const T* __restr
   }
 }
 
+// ---- sequence pooling + pooler head ---------------------------------------------------
+// One workgroup per (sequence, 8 chunks of 16 bytes): 32 token lanes stride over the sequence's
+// tokens, fp32 sum / max per column, combined through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void sequence_pool_kernel(const T* __restrict__ hidden,
+                                                            const int* __restrict__ seq_blocks,
+                                                            const int* __restrict__ seq_tokens, int width, int mode,
+                                                            T* __restrict__ out) {
+  constexpr int N = Vec<T>::N;
+  __shared__ float red[32][8 * N + 1];
+  const int s = blockIdx.x;
+  const int cw = threadIdx.x & 7, tl = threadIdx.x >> 3;
+  const int col = (blockIdx.y * 8 + cw) * N;
+  const int64_t t0 = int64_t(seq_blocks[s]) * 64;
+  int count = (seq_blocks[s + 1] - seq_blocks[s]) * 64;
+  if (seq_tokens) count = min(max(seq_tokens[s], 1), count);
+  int first = 0, last = count;
+  if (mode == RT_POOL_FIRST) last = 1;
+  else if (mode == RT_POOL_LAST) first = count - 1;
+  float acc[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) acc[i] = mode == RT_POOL_MAX ? -INFINITY : 0.f;
+  if (col < width)
+    for (int t = first + tl; t < last; t += 32) {
+      float x[N];
+      Vec<T>::load(hidden + (t0 + t) * width + col, x);
+#pragma unroll
+      for (int i = 0; i < N; ++i) acc[i] = mode == RT_POOL_MAX ? fmaxf(acc[i], x[i]) : acc[i] + x[i];
+    }
+#pragma unroll
+  for (int i = 0; i < N; ++i) red[tl][cw * N + i] = acc[i];
+  __syncthreads();
+  if (threadIdx.x < 8 * N) {
+    const int c = blockIdx.y * 8 * N + threadIdx.x;
+    float v = red[0][threadIdx.x];
+    for (int r = 1; r < 32; ++r) v = mode == RT_POOL_MAX ? fmaxf(v, red[r][threadIdx.x]) : v + red[r][threadIdx.x];
+    if (mode == RT_POOL_MEAN) v /= float(last - first);
+    if (c < width) out[int64_t(s) * width + c] = static_cast<T>(v);
+  }
+}
+
+// out[b, j] = tanh(bias[j] + sum_i x[b, i] * w[j, i]), weights as [out, in]: one wave per output column.
+template <typename T>
+__global__ __launch_bounds__(256) void pooler_dense_tanh_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                const T* __restrict__ bias, T* __restrict__ out,
+                                                                int batch, int d_in, int d_out) {
+  constexpr int N = Vec<T>::N;
+  const int lane = threadIdx.x & 63, j = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (j >= d_out) return;
+  const T* wr = w + int64_t(j) * d_in;
+  const float bj = float(bias[j]);
+  for (int b = 0; b < batch; ++b) {
+    const T* xr = x + int64_t(b) * d_in;
+    float acc = 0.f;
+    for (int c = lane * N; c < d_in; c += 64 * N) {
+      float a[N], v[N];
+      Vec<T>::load(wr + c, a);
+      Vec<T>::load(xr + c, v);
+#pragma unroll
+      for (int i = 0; i < N; ++i) acc = fmaf(a[i], v[i], acc);
+    }
+    acc = group_sum<64>(acc);
+    if (lane == 0) out[int64_t(b) * d_out + j] = static_cast<T>(tanhf(acc + bj));
+  }
+}
+
 int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "%s launch failed: %s", what, hipGetErrorString(e));
@@ -633,6 +699,47 @@ int rt_embed_layernorm(const int* input_ids, const int* position_ids, const int*
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "embed_layernorm launch failed: %s", hipGetErrorString(e));
   return RT_OK;
+}
+
+int rt_sequence_pool(const void* hidden, const int* seq_blocks_dev, const int* seq_tokens_dev, int batch, int width,
+                     int mode, void* out, int dtype, void* stream) {
+  RT_REQUIRE(hidden && seq_blocks_dev && out, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(batch >= 1 && batch <= 65535, RT_EINVAL, "batch=%d out of range [1, 65535]", batch);
+  RT_REQUIRE(width > 0 && width % 8 == 0, RT_EINVAL, "width=%d must be a positive multiple of 8", width);
+  RT_REQUIRE(mode == RT_POOL_FIRST || mode == RT_POOL_LAST || mode == RT_POOL_MEAN || mode == RT_POOL_MAX, RT_EINVAL,
+             "unknown pooling mode %d", mode);
+  RT_REQUIRE(aligned16(hidden), RT_EINVAL, "hidden must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto tag) {
+    typedef decltype(tag) T;
+    const int per_wg = 8 * Vec<T>::N;
+    hipLaunchKernelGGL(sequence_pool_kernel<T>, dim3(batch, (width + per_wg - 1) / per_wg), dim3(256), 0, st,
+                       (const T*)hidden, seq_blocks_dev, seq_tokens_dev, width, mode, (T*)out);
+  };
+  if (dtype == RT_F16) launch(__half());
+  else if (dtype == RT_BF16) launch(__hip_bfloat16());
+  else if (dtype == RT_F32) launch(float());
+  else return rt::fail(RT_EINVAL, "unknown dtype %d", dtype);
+  return check_launch("sequence_pool");
+}
+
+int rt_pooler_dense_tanh(const void* pooled, const void* weight_t, const void* bias, void* out, int batch, int d_in,
+                         int d_out, int dtype, void* stream) {
+  RT_REQUIRE(pooled && weight_t && bias && out, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(batch >= 1 && d_out >= 1, RT_EINVAL, "bad shape: batch=%d d_out=%d", batch, d_out);
+  RT_REQUIRE(d_in > 0 && d_in % 8 == 0, RT_EINVAL, "d_in=%d must be a positive multiple of 8", d_in);
+  RT_REQUIRE(aligned16(pooled) && aligned16(weight_t), RT_EINVAL, "pooled and weight_t must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  auto launch = [&](auto tag) {
+    typedef decltype(tag) T;
+    hipLaunchKernelGGL(pooler_dense_tanh_kernel<T>, dim3((d_out + 3) / 4), dim3(256), 0, st, (const T*)pooled,
+                       (const T*)weight_t, (const T*)bias, (T*)out, batch, d_in, d_out);
+  };
+  if (dtype == RT_F16) launch(__half());
+  else if (dtype == RT_BF16) launch(__hip_bfloat16());
+  else if (dtype == RT_F32) launch(float());
+  else return rt::fail(RT_EINVAL, "unknown dtype %d", dtype);
+  return check_launch("pooler_dense_tanh");
 }
 
 }  // extern "C"

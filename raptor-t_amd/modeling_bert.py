@@ -9,6 +9,7 @@ Differences: sizes are read from the weights (no 768 / 3072 literals), LayerNorm
 the dtype are arguments, and `from_weights` builds layers from plain tensors so that a
 random-init model needs no HuggingFace object.
 """
+import enum
 import os
 import sys
 from typing import Optional, Sequence
@@ -244,6 +245,85 @@ class BertModelNoPooler:
                                  BertEncoder.from_torch(model.encoder, async_, dtype, eps))
 
 
+class PoolingType(enum.Enum):
+    FIRST = "First"
+    LAST = "Last"
+    MEAN = "Mean"
+    MAX = "Max"
+
+
+PoolingMap = {PoolingType.FIRST: "First", PoolingType.LAST: "Last", PoolingType.MEAN: "Mean", PoolingType.MAX: "Max"}
+_POOL_CODE = {"First": capi.RT_POOL_FIRST, "Last": capi.RT_POOL_LAST, "Mean": capi.RT_POOL_MEAN, "Max": capi.RT_POOL_MAX}
+
+
+class SequencePool:
+    """One row per sequence of a packed batch: the first / last token's hidden state, or the mean / maximum over
+    the sequence's tokens.  The reference's class is a stub that returns its output argument
+    (python/modeling_bert.py:270-277); the modes are its PoolingType (:298-314)."""
+
+    def __init__(self, pooling_type="First"):
+        if isinstance(pooling_type, PoolingType):
+            pooling_type = PoolingMap[pooling_type]
+        if pooling_type not in _POOL_CODE:
+            raise ValueError("unknown pooling type %r" % (pooling_type,))
+        self.mode = _POOL_CODE[pooling_type]
+
+    def __call__(self, input_tensor, seq_position_info_tensor, output_tensor=None, seq_tokens=None):
+        batch = seq_position_info_tensor.numel() - 1
+        if output_tensor is None:
+            output_tensor = torch.empty(batch, input_tensor.shape[1], dtype=input_tensor.dtype, device=input_tensor.device)
+        return capi.sequence_pool(input_tensor, seq_position_info_tensor, self.mode, output_tensor, seq_tokens)
+
+
+class BertPooler:
+    """tanh(dense(pooled)): the BertPooler the reference has commented out (python/modeling_bert.py:279-296);
+    weight arrives as [in, out] like every weight of the layers and is kept [out, in]."""
+
+    def __init__(self, weight, bias):
+        if weight.dim() != 2 or bias.numel() != weight.shape[1]:
+            raise ValueError("BertPooler: weight must be [in, out] and bias [out]")
+        self.weight_t = weight.t().contiguous().cuda()
+        self.bias = bias.contiguous().cuda()
+
+    def __call__(self, input_tensor, output=None):
+        if output is None:
+            output = torch.empty(input_tensor.shape[0], self.weight_t.shape[0], dtype=input_tensor.dtype,
+                                 device=input_tensor.device)
+        return capi.pooler_dense_tanh(input_tensor, self.weight_t, self.bias, output)
+
+    @staticmethod
+    def from_torch(pooler, bigbird: bool = True, dtype=torch.float16):
+        """pooler: BigBirdModel.pooler (an nn.Linear; bigbird=True) or BertModel.pooler (with .dense)."""
+        lin = pooler if bigbird else pooler.dense
+        return BertPooler(torch.t(lin.weight.detach()).contiguous().to(dtype), lin.bias.detach().to(dtype))
+
+
+class BertModel:
+    """BertModelNoPooler + SequencePool + BertPooler (python/modeling_bert.py:398-440, whose from_torch leaves the
+    pooler out): returns (sequence_output, pooler_output, test_info)."""
+
+    def __init__(self, model_nopooler, pooler):
+        self.bertmodel_nopooler = model_nopooler
+        self.pooler = pooler
+
+    def __call__(self, inputs, total_seq_len, thread_block_limit, seq_position_info, seq_position_info_tensor,
+                 partition_part_index_tensor, partition_part_tensor, pooling_type=PoolingType.FIRST,
+                 pooler_output=None, **kwargs):
+        sequence_output, test_info = self.bertmodel_nopooler(
+            inputs, total_seq_len, thread_block_limit, seq_position_info, seq_position_info_tensor,
+            partition_part_index_tensor, partition_part_tensor, **kwargs)
+        pooled = SequencePool(pooling_type)(sequence_output, seq_position_info_tensor,
+                                            seq_tokens=kwargs.get("attention_masks"))
+        return sequence_output, self.pooler(pooled, pooler_output), test_info
+
+    @staticmethod
+    def from_torch(model, async_: bool = True, dtype=torch.float16, eps=None, bigbird: bool = True):
+        if getattr(model, "pooler", None) is None:
+            raise ValueError("the torch model was built without a pooling layer")
+        return BertModel(BertModelNoPooler.from_torch(model, async_, dtype, eps),
+                         BertPooler.from_torch(model.pooler, bigbird, dtype))
+
+
 def _model_from_checkpoint(path, heads=None, async_=True, dtype=torch.float16, eps=None, device="cuda"):
     emb, layers, cfg = checkpoint.load(path)
     heads = cfg.get("num_attention_heads") if heads is None else heads
@@ -260,6 +340,17 @@ def _model_from_checkpoint(path, heads=None, async_=True, dtype=torch.float16, e
     return BertModelNoPooler(embeddings, BertEncoder.from_weights([dev(w) for w in layers], heads, async_, eps))
 
 
+def _model_with_pooler_from_checkpoint(path, heads=None, async_=True, dtype=torch.float16, eps=None, device="cuda"):
+    """BertModel from a checkpoint on disk that holds a pooling head (see BertModelNoPooler.from_local_checkpoint)."""
+    sd, _ = checkpoint.read_state_dict(path)
+    head = checkpoint.pooler_from_state_dict(sd)
+    if head is None:
+        raise KeyError("the checkpoint has no pooler.weight / pooler.dense.weight")
+    weight, bias = (t.detach().to(device=device, dtype=dtype) for t in head)
+    return BertModel(_model_from_checkpoint(path, heads, async_, dtype, eps, device), BertPooler(weight, bias))
+
+
+BertModel.from_local_checkpoint = staticmethod(_model_with_pooler_from_checkpoint)
 BertModelNoPooler.from_local_checkpoint = staticmethod(_model_from_checkpoint)
 BertModelNoPooler.from_local_checkpoint.__doc__ = (
     "Builds the model from a HuggingFace BigBird / BERT checkpoint on disk (a directory with config.json and "

@@ -28,8 +28,20 @@ def hf_state_dict(hidden=16, ffn=24, layers=2, prefix="", seed=0):
         sd[b + "output.dense.weight"], sd[b + "output.dense.bias"] = r(hidden, ffn), r(hidden)
         for ln in ("attention.output.LayerNorm", "output.LayerNorm"):
             sd[b + ln + ".weight"], sd[b + ln + ".bias"] = r(hidden), r(hidden)
-    sd[prefix + "pooler.weight"] = r(hidden, hidden)           # ignored
+    sd[prefix + "pooler.weight"] = r(hidden, hidden)           # ignored by convert_state_dict
     return sd
+
+
+def test_pooler_head_is_found_in_both_spellings():
+    sd = hf_state_dict(prefix="bert.")
+    assert ck.pooler_from_state_dict(sd) is None               # a weight without its bias is not a head
+    sd["bert.pooler.bias"] = torch.arange(16.0)
+    w, b = ck.pooler_from_state_dict(sd)
+    x = torch.randn(3, 16)
+    assert torch.allclose(x @ w + b, torch.nn.functional.linear(x, sd["bert.pooler.weight"], sd["bert.pooler.bias"]))
+    bert = {k.replace("pooler.", "pooler.dense."): v for k, v in sd.items()}
+    w2, b2 = ck.pooler_from_state_dict(bert)
+    assert torch.equal(w, w2) and torch.equal(b, b2)
 
 
 @pytest.mark.parametrize("prefix", ["", "bert."])

@@ -305,6 +305,48 @@ def test_gemm_exhaustive_tuning_keeps_results(capi):
     gemm.close()
 
 
+@pytest.mark.parametrize("dtype,width", [(torch.float16, 768), (torch.bfloat16, 1024), (torch.float32, 200)])
+def test_sequence_pool_matches_oracle(capi, dtype, width):
+    say("sequence pool", dtype, width)
+    g = torch.Generator().manual_seed(9)
+    seq_lens = [64 * 5, 64, 64 * 33, 64 * 2]
+    sb = capi.seq_prefix_blocks(seq_lens)
+    sb_d = torch.from_numpy(sb).cuda()
+    hidden = torch.randn(sum(seq_lens), width, generator=g).to(dtype).cuda()
+    tokens = [300, 1, 64 * 33 - 63, 128]
+    tok_d = torch.tensor(tokens, dtype=torch.int32).cuda()
+    tol = 1e-5 if dtype == torch.float32 else (2e-3 if dtype == torch.float16 else 1.6e-2)
+    for name, code in (("First", capi.RT_POOL_FIRST), ("Last", capi.RT_POOL_LAST), ("Mean", capi.RT_POOL_MEAN),
+                       ("Max", capi.RT_POOL_MAX)):
+        for toks, toks_d in ((None, None), (tokens, tok_d)):
+            out = torch.full((4, width), float("nan"), dtype=dtype, device="cuda")
+            capi.sequence_pool(hidden, sb_d, code, out, toks_d)
+            torch.cuda.synchronize()
+            want = ol.sequence_pool(hidden.float().cpu(), sb.tolist(), name, seq_tokens=toks)
+            err = (out.float().cpu() - want).abs().max().item()
+            assert err <= tol, (name, toks is not None, err)
+            if name in ("First", "Last", "Max"):               # selections: the stored values themselves
+                assert torch.equal(out.float().cpu(), want)
+    with pytest.raises(capi.RaptorError):
+        capi.sequence_pool(hidden, sb_d, 7, out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_pooler_dense_tanh_matches_oracle(capi, dtype):
+    say("pooler", dtype)
+    g = torch.Generator().manual_seed(10)
+    for batch, d_in, d_out in ((16, 768, 768), (3, 200, 50), (1, 8, 1)):
+        x = torch.randn(batch, d_in, generator=g).to(dtype).cuda()
+        w = (torch.randn(d_in, d_out, generator=g) * 0.05).to(dtype).cuda()
+        b = torch.randn(d_out, generator=g).to(dtype).cuda()
+        out = torch.full((batch, d_out), float("nan"), dtype=dtype, device="cuda")
+        capi.pooler_dense_tanh(x, w.t().contiguous(), b, out)
+        torch.cuda.synchronize()
+        want = ol.pooler(x.float().cpu(), w.float().cpu(), b.float().cpu())
+        tol = 1e-5 if dtype == torch.float32 else (1e-3 if dtype == torch.float16 else 8e-3)
+        assert (out.float().cpu() - want).abs().max().item() <= tol
+
+
 @pytest.mark.parametrize("retune", [0, 3, 8])
 def test_gemm_retuning_for_new_token_counts_keeps_results(capi, retune):
     """A new M of a kind already tuned times `retune` of the kind's best solutions (or none): same results."""

@@ -179,6 +179,52 @@ def test_from_torch_matches_huggingface_bigbird(mb, ut, length):
     assert err <= 2e-2
 
 
+def test_model_with_pooler_matches_huggingface_bigbird(mb, ut, tmp_path):
+    """BertModel (encoder + SequencePool(First) + BertPooler) against HuggingFace BigBirdModel's
+    last_hidden_state and pooler_output."""
+    say("hf pooler")
+    from transformers import BigBirdConfig, BigBirdModel
+    torch.manual_seed(1)
+    length = 832
+    cfg = BigBirdConfig(vocab_size=1000, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        intermediate_size=256, max_position_embeddings=4096, attention_type="block_sparse",
+                        block_size=64, num_random_blocks=3, hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+    hf = BigBirdModel(cfg, add_pooling_layer=True).cuda().train()
+    ids = torch.randint(1, 1000, (1, length), device="cuda")
+    with torch.no_grad():
+        ref = hf(input_ids=ids)
+    model = mb.BertModel.from_torch(hf, async_=True, dtype=torch.float16)
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo([length], 64, 48, 2)
+    meta.update_meta_data(length, spi[-1] + 1, total_comp, spi)
+    pos = torch.arange(length, device="cuda")
+    inter = torch.empty(length, 256, dtype=torch.float16, device="cuda")
+    seq, pooled, _ = model(ids[0], length, 48, spi, spi_t, ppi_t, pp_t, token_type_ids=torch.zeros_like(pos),
+                           position_ids=pos, intermediate_temp=inter)
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    assert (seq.float().cpu() - ref.last_hidden_state[0].float().cpu()).abs().max().item() <= 2e-2
+    assert tuple(pooled.shape) == (1, 128)
+    err = (pooled.float().cpu() - ref.pooler_output.float().cpu()).abs().max().item()
+    say("  pooler err", err)
+    assert err <= 2e-2
+    with pytest.raises(ValueError):
+        mb.BertModel.from_torch(BigBirdModel(cfg, add_pooling_layer=False), dtype=torch.float16)
+    with pytest.raises(ValueError):
+        mb.SequencePool("Median")
+    # the same model through a checkpoint on disk
+    hf.save_pretrained(str(tmp_path), safe_serialization=True)
+    disk = mb.BertModel.from_local_checkpoint(str(tmp_path), async_=True, dtype=torch.float16)
+    meta = mb.cxx.MetaData()
+    meta.update_meta_data(length, spi[-1] + 1, total_comp, spi)
+    _, pooled2, _ = disk(ids[0], length, 48, spi, spi_t, ppi_t, pp_t, token_type_ids=torch.zeros_like(pos),
+                         position_ids=pos, intermediate_temp=inter)
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    assert torch.equal(pooled2, pooled)
+
+
 def test_local_checkpoint_matches_huggingface_bigbird(mb, ut, tmp_path):
     """A HuggingFace BigBird checkpoint written to disk (safetensors + config.json), read back by
     from_local_checkpoint, against the HuggingFace model that wrote it."""

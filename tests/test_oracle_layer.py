@@ -1,6 +1,7 @@
 """Layer glue and epilogues of the oracle against library routines."""
 import math
 
+import pytest
 import torch
 import torch.nn.functional as F
 
@@ -78,3 +79,33 @@ def test_embeddings_layernorm_matches_torch_modules_and_hand_case():
     out = ol.embeddings_layernorm(torch.tensor([0]), torch.tensor([0]), torch.tensor([0]), w, p, ty,
                                   torch.tensor([2.0, 3.0]), torch.tensor([0.5, -0.5]), eps=0.0)
     assert torch.allclose(out, torch.tensor([[-1.5, 2.5]]), atol=1e-6)
+
+
+def test_sequence_pool_and_pooler_match_torch_and_hand_cases():
+    """sequence_pool against per-sequence torch reductions written out here and a hand case; pooler against
+    torch's own Linear + Tanh modules (HuggingFace BigBirdModel: activation(pooler(sequence_output[:, 0])))."""
+    g = torch.Generator().manual_seed(8)
+    seq_blocks = [0, 2, 3, 6]
+    hidden = torch.randn(6 * 64, 16, generator=g)
+    tokens = [100, 64, 131]
+    for mode, fn in (("First", lambda x: x[0]), ("Last", lambda x: x[-1]), ("Mean", lambda x: x.mean(0)),
+                     ("Max", lambda x: x.amax(0))):
+        full = ol.sequence_pool(hidden, seq_blocks, mode)
+        cut = ol.sequence_pool(hidden, seq_blocks, mode, seq_tokens=tokens)
+        for s in range(3):
+            t0, n = seq_blocks[s] * 64, (seq_blocks[s + 1] - seq_blocks[s]) * 64
+            assert torch.allclose(full[s], fn(hidden[t0:t0 + n]), atol=1e-6)
+            assert torch.allclose(cut[s], fn(hidden[t0:t0 + tokens[s]]), atol=1e-6)
+    ramp = torch.arange(64, dtype=torch.float32)[:, None].repeat(1, 2)
+    assert ol.sequence_pool(ramp, [0, 1], "Mean").tolist() == [[31.5, 31.5]]
+    assert ol.sequence_pool(ramp, [0, 1], "Last", seq_tokens=[10]).tolist() == [[9.0, 9.0]]
+    with pytest.raises(ValueError):
+        ol.sequence_pool(ramp, [0, 1], "Median")
+    lin = torch.nn.Linear(16, 12)
+    x = torch.randn(5, 16, generator=g)
+    with torch.no_grad():
+        want = torch.tanh(lin(x))
+        got = ol.pooler(x, lin.weight.t().contiguous(), lin.bias)
+    assert (got - want).abs().max().item() <= 1e-6
+    one = ol.pooler(torch.tensor([[1.0, 2.0]]), torch.tensor([[0.5], [0.25]]), torch.tensor([-1.0]))
+    assert abs(one.item() - 0.0) < 1e-7                       # tanh(0.5 + 0.5 - 1)
