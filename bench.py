@@ -177,10 +177,18 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
     return out
 
 
-def time_kernel(fn, steps, warmup):
+def time_kernel(fn, steps, warmup, settle_ms=25.0):
+    """Median duration of one launch in microseconds.  After the warm-up launches the kernel keeps running
+    for `settle_ms`: from idle the GPU takes some tens of launches to reach its sustained clocks (the first
+    launches of a 100 us kernel measure 10-15 % slow), and a kernel inside a running job never sees that ramp."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for a, b in evs:
         a.record()

@@ -24,9 +24,9 @@
 //
 // Softmax is evaluated in base 2 (q arrives pre-multiplied by log2(e)/sqrt(d)).  The S^T
 // accumulator starts at minus the row's reference maximum, so the MFMA result feeds exp2
-// directly; the reference is only moved (and O, l rescaled) when some P = 2^(score -
-// reference) exceeds 2^6, detected on the packed 16-bit P values: a rare, wave-uniform
-// branch that recomputes the half tile with a proper maximum.
+// directly; the reference is only moved (and O, l rescaled) when a lane's partial row sum of
+// P = 2^(score - reference) over one key tile exceeds 2^11: a rare, wave-uniform branch that
+// recomputes the half tile with a proper maximum.
 //
 // The kernel is persistent (two workgroups per CU).  Without a plan it makes its own
 // schedule: global rows first, each XCD (one L2 per XCD; workgroups are dealt round-robin to
@@ -48,13 +48,9 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
-
-__device__ inline uint32_t pk_max_u16(uint32_t a, uint32_t b) {
-  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
-}
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
@@ -64,24 +60,15 @@ template <> struct Mma<_Float16> {
   // a[0..7] = p[0..7] rounded to T; returns the fp32 sum of the ROUNDED values (what PV multiplies)
   __device__ static float pack(const float* p, v8& out) {
     float s = 0.f;
+    u32x4 w;                                  // whole dwords: each pair stays one v_cvt_pk_f16_f32
 #pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-      f16x2 h = {static_cast<_Float16>(p[e]), static_cast<_Float16>(p[e + 1])};
-      out[e] = h[0];
-      out[e + 1] = h[1];
+    for (int i = 0; i < 4; ++i) {
+      const f16x2 h = __builtin_convertvector(f32x2{p[2 * i], p[2 * i + 1]}, f16x2);
+      w[i] = __builtin_bit_cast(uint32_t, h);
       s = __builtin_amdgcn_fdot2(h, f16x2{1, 1}, s, false);
     }
+    out = __builtin_bit_cast(v8, w);
     return s;
-  }
-  // positive halves order like unsigned 16-bit integers: running packed maximum of the bit patterns
-  __device__ static uint32_t max_bits(const v8& p, uint32_t acc) {
-    const u32x4 w = __builtin_bit_cast(u32x4, p);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc = pk_max_u16(acc, w[i]);
-    return acc;
-  }
-  __device__ static bool over_threshold(uint32_t top) {      // 64.0 in fp16 is 0x5400
-    return (top & 0xffffu) > 0x5400u || (top >> 16) > 0x5400u;
   }
 };
 template <> struct Mma<__bf16> {
@@ -96,19 +83,13 @@ template <> struct Mma<__bf16> {
     for (int e = 0; e < 8; ++e) out[e] = static_cast<__bf16>(p[e]);
     return ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
   }
-  __device__ static uint32_t max_bits(const v8& p, uint32_t acc) {
-    const u32x4 w = __builtin_bit_cast(u32x4, p);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc = pk_max_u16(acc, w[i]);
-    return acc;
-  }
-  __device__ static bool over_threshold(uint32_t top) {      // 64.0 in bf16 is 0x4280
-    return (top & 0xffffu) > 0x4280u || (top >> 16) > 0x4280u;
-  }
 };
 
-// A row's reference maximum only moves when some P = 2^(score - reference) would exceed 2^6
-// (tested on the packed 16-bit P values; see over_threshold).
+// A row's reference maximum only moves when the 32 values P = 2^(score - reference) a lane holds
+// for one key tile add up to more than 2^11 (no single P can then exceed 2^11, far inside fp16's
+// range, and P keeps its full relative precision at any magnitude): the row sum the kernel needs
+// anyway doubles as the overflow test.
+constexpr float SUM_LIMIT = 2048.0f;
 
 // Online-softmax state of one wave for its 64 queries: O^T as [d tile][query tile].
 struct State {
@@ -189,21 +170,19 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
         }
       };
       // exp2 of the (already shifted) scores -> P as the B operand of the second product:
-      // step s takes accumulator registers 8*(s&1)..+7 of key tile s>>1.  Returns true when
-      // some P exceeds 2^RESCALE_THRESHOLD (or is not finite).
+      // step s takes accumulator registers 8*(s&1)..+7 of key tile s>>1.  Returns true when the
+      // lane's 32 values of P add up to more than SUM_LIMIT (or to something not finite).
       auto exponentiate = [&]() {
         float part[4];
-        uint32_t top = 0;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
           float p8[8];
 #pragma unroll
           for (int e = 0; e < 8; ++e) p8[e] = __builtin_amdgcn_exp2f(sc[s >> 1][8 * (s & 1) + e]);
           part[s] = Mma<T>::pack(p8, pb[s]);
-          top = Mma<T>::max_bits(pb[s], top);
         }
         psum = (part[0] + part[1]) + (part[2] + part[3]);
-        return Mma<T>::over_threshold(top);
+        return !(psum <= SUM_LIMIT);                    // also true for an infinite or undefined sum
       };
       bool redo = fresh;
       if (!fresh) {
