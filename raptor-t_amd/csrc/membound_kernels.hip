@@ -92,12 +92,21 @@ __global__ __launch_bounds__(256) void bias_residual_layernorm_kernel(
   const T* r = residual + row * HIDDEN;
   float x[CHUNKS][N];
   float sum = 0.f;
+  // every request of the row goes out before the first conversion waits for one (left to itself
+  // the compiler serialises them for some CHUNKS)
+  uint4 ra[CHUNKS], rr[CHUNKS];
+#pragma unroll
+  for (int c = 0; c < CHUNKS; ++c) {
+    const int col = (c * G + lane) * N;
+    ra[c] = *reinterpret_cast<const uint4*>(o + col);
+    rr[c] = *reinterpret_cast<const uint4*>(r + col);
+  }
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) {
     const int col = (c * G + lane) * N;
     float a[N], b[N], d[N];
-    Vec<T>::load(o + col, a);
-    Vec<T>::load(r + col, b);
+    Vec<T>::load(reinterpret_cast<const T*>(&ra[c]), a);
+    Vec<T>::load(reinterpret_cast<const T*>(&rr[c]), b);
     Vec<T>::load(bias + col, d);
 #pragma unroll
     for (int i = 0; i < N; ++i) { x[c][i] = a[i] + d[i] + b[i]; sum += x[c][i]; }
