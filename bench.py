@@ -108,6 +108,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
 
     mb.cxx.set_gemm_epilogue_fusion(not args.no_epilogue_fusion)
     mb.cxx.set_attention_q_from_rows(not args.materialize_q)
+    mb.cxx.set_attention_host_plan(args.lpt_plan)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -293,6 +294,7 @@ def run_streaming(args):
         enc(h, t, args.block_limit, spi, spi_t, ppi_t, pp_t, tmp[:t], inter[:t], attn[:t], test_info={},
             balanced=args.lpt_plan)
 
+    mb.cxx.set_attention_host_plan(args.lpt_plan)
     # Start-up tuning, as a server does once: the GEMMs of every token count the batches can have (16 sequences of
     # 512..4096 tokens in steps of 64).  Without it the first batch of each token count stalls ~17 ms on timing
     # six candidate kernels per GEMM; --no-pretune shows that.

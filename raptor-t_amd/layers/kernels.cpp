@@ -140,8 +140,11 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
 namespace {
 std::atomic<bool> g_epilogue_fusion{true};
 std::atomic<bool> g_q_from_rows{true};
+std::atomic<bool> g_host_plan{false};
 constexpr float kQScale = 1.4426950408889634f / 8.0f;      // log2(e) / sqrt(64): the softmax runs in base 2
 }
+void set_attention_host_plan(bool on) { g_host_plan.store(on); }
+bool attention_host_plan() { return g_host_plan.load(); }
 void set_attention_q_from_rows(bool on) { g_q_from_rows.store(on); }
 bool attention_q_from_rows() { return g_q_from_rows.load(); }
 void set_gemm_epilogue_fusion(bool on) { g_epilogue_fusion.store(on); }
@@ -291,9 +294,11 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
       throw std::invalid_argument("balanced attention: the plan has a different number of workgroups than block_limit");
     if (from_select_index.numel() != int64_t(block_num) * head_num)
       throw std::invalid_argument("balanced attention: the plan does not cover every (head, block) unit");
-    from_idx = from_select_index.data_ptr<int>();
-    from_pos = from_select_index_position.data_ptr<int>();
-    n_wg = block_limit;
+    if (attention_host_plan()) {
+      from_idx = from_select_index.data_ptr<int>();
+      from_pos = from_select_index_position.data_ptr<int>();
+      n_wg = block_limit;
+    }
   }
   if (qkv_rows.defined()) {
     require_cuda_contiguous(qkv_rows, "qkv_rows");

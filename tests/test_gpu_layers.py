@@ -61,6 +61,7 @@ def test_encoder_through_layer_api_matches_oracle(mb, ut, async_, balanced, dtyp
     enc = mb.BertEncoder.from_weights(layers_w, heads, async_=async_, eps=eps)
     meta = mb.cxx.MetaData()
     worst = 0.0
+    mb.cxx.set_attention_host_plan(balanced)               # balanced: walk the host's LPT partition, as the reference does
     for seq_lens in ([832, 1024, 256], [1280, 768]):       # two batches through the same objects
         t = sum(seq_lens)
         x32 = torch.randn(t, hidden, generator=g)
@@ -79,6 +80,7 @@ def test_encoder_through_layer_api_matches_oracle(mb, ut, async_, balanced, dtyp
         err = (out.float().cpu() - want).abs().max().item()
         say("  err", err, "info", info)
         worst = max(worst, err)
+    mb.cxx.set_attention_host_plan(False)
     meta.terminate_thread()
     assert worst <= (2e-2 if dtype == torch.float16 else 8e-2)   # bf16: one ulp at |y| ~ 4 is 3e-2
 
@@ -118,6 +120,34 @@ def test_fused_and_unfused_paths_agree(mb, ut):
     meta.terminate_thread()
     assert (outs[0] - outs[1]).abs().max().item() <= 2e-2
     assert (outs[0] - outs[2]).abs().max().item() <= 2e-2
+
+
+def test_balanced_launch_schedules_give_the_same_bits(mb, ut):
+    """balanced=True with the kernel's own schedule (the default), balanced=True walking the host's LPT partition
+    and balanced=False compute every unit the same way: identical outputs."""
+    say("balanced schedules")
+    hidden, heads, ffn, dtype = 768, 12, 3072, torch.float16
+    g = torch.Generator().manual_seed(3)
+    w = {k: v.to(dtype).cuda() for k, v in ol.random_layer_weights(hidden, ffn, g).items()}
+    layer = mb.BertLayer.from_weights(w, heads, 0, async_=True)
+    meta = mb.cxx.MetaData()
+    seq_lens = [1408, 192, 832]
+    t = sum(seq_lens)
+    x = torch.randn(t, hidden, generator=g).to(dtype).cuda()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, 64, heads)
+    assert not mb.cxx.attention_host_plan()
+    outs = []
+    for balanced, host_plan in ((True, False), (True, True), (False, False)):
+        mb.cxx.set_attention_host_plan(host_plan)
+        meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+        new = lambda wd: torch.empty(t, wd, dtype=dtype, device="cuda")
+        out, _ = layer(x.clone(), spi, spi_t, ppi_t, pp_t, new(ffn), new(hidden), new(hidden), 64, balanced=balanced)
+        torch.cuda.synchronize()
+        outs.append(out.clone())
+    mb.cxx.set_attention_host_plan(False)
+    meta.terminate_thread()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert not torch.isnan(outs[0]).any()
 
 
 def test_startup_gemm_tuning_runs(mb):
@@ -295,6 +325,7 @@ def test_padded_sequence_matches_huggingface_with_attention_mask(mb, ut, length,
     meta.update_meta_data(length, spi[-1] + 1, total_comp, spi)
     inter = torch.empty(length, 256, dtype=torch.float16, device="cuda")
     for balanced in (True, False):
+        mb.cxx.set_attention_host_plan(balanced)
         out, _ = model(p["input_ids"], length, 48, spi, spi_t, ppi_t, pp_t, attention_masks=p["seq_tokens_tensor"],
                        token_type_ids=p["token_type_ids"], position_ids=p["position_ids"], intermediate_temp=inter,
                        balanced=balanced)
