@@ -122,6 +122,35 @@ def test_fused_and_unfused_paths_agree(mb, ut):
     assert (outs[0] - outs[2]).abs().max().item() <= 2e-2
 
 
+def test_batches_of_changing_geometry_back_to_back(mb, ut):
+    """Eight batches of different geometry enqueued without a synchronisation in between (the index workers run
+    ahead, the slots of the block-index pipeline are reused every second batch): every batch matches the oracle."""
+    say("changing geometry")
+    hidden, heads, ffn, dtype, eps = 256, 4, 512, torch.float16, 1e-5
+    g = torch.Generator().manual_seed(7)
+    layers_w32 = [ol.random_layer_weights(hidden, ffn, g) for _ in range(3)]
+    layers_w = [{k: v.to(dtype).cuda() for k, v in w.items()} for w in layers_w32]
+    enc = mb.BertEncoder.from_weights(layers_w, heads, async_=True, eps=eps)
+    meta = mb.cxx.MetaData()
+    batches = [[832, 64], [128], [1024, 256, 192], [64, 64, 64, 64], [896], [768, 832], [320, 1216], [64]]
+    runs = []
+    for seq_lens in batches:
+        t = sum(seq_lens)
+        x32 = torch.randn(t, hidden, generator=g)
+        hs = x32.to(dtype).cuda()
+        spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, 32, heads)
+        meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+        new = lambda w: torch.empty(t, w, dtype=dtype, device="cuda")
+        out, _ = enc(hs, t, 32, spi, spi_t, ppi_t, pp_t, new(hidden), new(ffn), new(hidden), test_info={})
+        runs.append((seq_lens, x32, out))                 # no synchronisation: the next batch is published at once
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    for seq_lens, x32, out in runs:
+        want = _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype)
+        err = (out.float().cpu() - want).abs().max().item()
+        assert err <= 2e-2, (seq_lens, err)
+
+
 def test_balanced_launch_schedules_give_the_same_bits(mb, ut):
     """balanced=True with the kernel's own schedule (the default), balanced=True walking the host's LPT partition
     and balanced=False compute every unit the same way: identical outputs."""
