@@ -1,0 +1,44 @@
+"""Host-side checks of bench.py that need no GPU: the one-GPU rule, the pair count behind the attention FLOPs
+and the roofline helpers."""
+import importlib.util
+import json
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _bench():
+    spec = importlib.util.spec_from_file_location("rt_bench", os.path.join(ROOT, "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "one gpu" in (r.stdout + r.stderr).lower()
+
+
+def test_block_pairs_follow_the_bigbird_row_rules():
+    """10n - 18 key blocks per (sequence, head) for a sparse sequence (two dense rows of n, two rows of 7, the
+    others 8), n*n below twelve blocks: the figure the attention FLOPs are derived from."""
+    b = _bench()
+    for n in (12, 13, 64):
+        rows = [n, 7] + [8] * (n - 4) + [7, n]
+        assert sum(rows) == 10 * n - 18
+        assert b.block_pairs([0, n], 3) == 3 * (10 * n - 18)
+    assert b.block_pairs([0, 5, 16], 2) == 2 * (25 + 11 * 11)
+    assert b.block_pairs([0, 64] + [64 * i for i in range(2, 9)], 12) == 59712        # config 2
+    assert b.PAIR_FLOP == 4 * 64 * 64 * 64
+
+
+def test_hbm_roofline_arithmetic():
+    b = _bench()
+    r = b.hbm_roofline("k", 8_000_000, 2.0, traffic=9e6)
+    assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0
+    assert abs(r["achieved"] - 4000.0) < 1e-9 and abs(r["frac"] - 0.5) < 1e-12
+    assert r["traffic"] == 9e6 and r["bytes_per_launch"] == 8_000_000
+    json.dumps(r)
