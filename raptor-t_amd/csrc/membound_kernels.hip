@@ -398,9 +398,9 @@ __global__ __launch_bounds__(256) void bias_gelu_kernel(T* __restrict__ out, con
 }
 
 // ---- QKV bias + scale + head split --------------------------------------------------------
-// Workgroup (g, h): global block g, head h.  The three 64x64 tiles are staged in LDS (bias
-// and scale applied) and written out in MFMA "fragment order": a tile is 8 fragments of
-// 64 lanes x 8 elements, element e of lane l of fragment f being
+// Workgroup (g, h): global block g, head h.  Its 64x64 tiles (bias and, for Q, the scale applied)
+// are written out in MFMA "fragment order": a tile is 8 fragments of 64 lanes x 8 elements,
+// element e of lane l of fragment f being
 //     Q, K :  tile[32*(f>>2) + (l&31)][16*(f&3) + 8*(l>>5) + e]        (row = token, col = d)
 //     V    :  tile[token(16*(f&3) + 8*(l>>5) + e)][32*(f>>2) + (l&31)] (transposed; token()
 //             swaps bits 2 and 3 of the slot index: the order in which a 32x32 accumulator
