@@ -83,6 +83,11 @@ def test_qkv_bias_split_layout_bit_exact(capi, dtype):
         flat = torch.empty(t, dm, dtype=dtype, device="cuda")
         capi.unpack_head_tiles(packed, flat, torch.from_numpy(sb).cuda(), heads, tr)
         assert torch.equal(flat.cpu().view(t, heads, 64), rnd(want))
+    # without a Q output (the attention kernel then reads its queries from `qkv`): K and V^T unchanged
+    k2, vt2 = (torch.full((t * dm,), float("nan"), dtype=dtype, device="cuda") for _ in range(2))
+    capi.qkv_bias_split(qkv, bias, None, k2, vt2, torch.from_numpy(sb).cuda(), heads, 0.125)
+    torch.cuda.synchronize()
+    assert torch.equal(k2, k) and torch.equal(vt2, vt)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
