@@ -5,40 +5,54 @@
 //
 // One wave owns all 64 queries of a unit and streams K / V^T tiles straight from global
 // memory into MFMA operand registers: the QKV split kernel stores every 64x64 tile in
-// "fragment order" (8 fragments of 64 lanes x 16 bytes), so each operand load is one fully
-// coalesced 1 KiB request and the main loop needs no LDS and no barrier.  The next K tile
-// is requested as soon as the last QK^T product of the current tile has issued, the next
-// V^T tile after the last PV product: one register copy of each, latency covered by the
-// softmax and the other product.
-//
-//   sparse rows : one wave per unit, 4 units (adjacent from-blocks) per workgroup
-//   global rows : the 4 waves of a workgroup take every 4th key block of ONE unit and merge
-//                 their online-softmax states through LDS at the end
+// "fragment order" (8 fragments of 64 lanes x 16 bytes), so each operand request is one fully
+// coalesced 1 KiB buffer load and the tile loop needs no LDS and no barrier.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_{f16,bf16}, fp32 accumulators):
 //   S^T[key][query] = K[key][:] . Q[query][:]       A = K fragment,   B = Q fragment
 //   O^T[d][query]  += V^T[d][key] . P^T[key][query]  A = V^T fragment, B = P (registers)
 // Both products put the query on the accumulator column (lane & 31): max, sum and rescale
 // factors are per-lane scalars and the S^T accumulators, after exp2, are the B operand of
-// the second product, so P never leaves registers.
+// the second product, so P never leaves registers.  Softmax is evaluated in base 2 (q arrives
+// pre-multiplied by log2(e)/sqrt(d)).
 //
-// Softmax is evaluated in base 2 (q arrives pre-multiplied by log2(e)/sqrt(d)).  The S^T
-// accumulator starts at minus the row's reference maximum, so the MFMA result feeds exp2
-// directly; the reference is only moved (and O, l rescaled) when a lane's partial row sum of
-// P = 2^(score - reference) over one key tile exceeds 2^11: a rare, wave-uniform branch that
-// recomputes the half tile with a proper maximum.
+// Two tile loops:
+//   pipelined (common path)  a (64 query x 64 key) tile is four 32x32 accumulator tiles
+//       a = (key half, query half); step j issues, one matrix instruction per handful of
+//       vector instructions, S^T(a[j+1]) and O^T += V^T P^T(a[j-1]) on the matrix pipe while
+//       the vector pipe turns S^T(a[j]) into P^T(a[j]).  The reference maximum is fixed per row
+//       (maximum over the row's first 32 keys, shared by a lane's two queries) and enters the
+//       score product as the MFMA's C operand.  Nothing is tested inside the loop: a row whose
+//       scores outgrow the reference shows up as a row sum that is not finite.
+//   moving maximum (fallback) such rows, rows of more than 64 entries per wave and launches with
+//       padded sequences are put aside and run afterwards by the loop that tracks the maximum
+//       tile by tile.  The two loops never share a loop nest: the register allocator treats
+//       them apart, and the pipelined one stays free of scratch-memory traffic.
 //
-// The kernel is persistent (two workgroups per CU).  Without a plan it makes its own
-// schedule: global rows first, each XCD (one L2 per XCD; workgroups are dealt round-robin to
-// the 8 XCDs) walking its own contiguous share of the (sequence, head) groups, so a group's
-// K/V tiles stay in one L2.  With an LPT plan, n_wg workgroups walk their unit lists.
+// Schedule: persistent workgroups (two per CU) that draw work from ticket counters in device
+// memory, one pair of counters per XCD (workgroups are dealt round-robin to the 8 XCDs, and each
+// XCD has its own L2): XCD x owns the x-th eighth of the (head, row) items, so the K / V^T tiles
+// of a (sequence, head) are fetched into one L2.
+//   phase 1  global rows (the first and last block of a sparse sequence): one workgroup per row,
+//            its 4 waves take every 4th key block and merge their softmax states through LDS;
+//            the two rows of a (sequence, head) are consecutive tickets, so they stream the
+//            same tiles at the same time;
+//   phase 2  all other rows: every wave draws single units.  While it computes unit u it knows
+//            unit u+1 (ticket, CSR row bounds and block ids through scalar loads), requests
+//            u+1's first K / V^T tile in u's last tile steps and u+1's queries in the same
+//            steps, and draws the ticket of unit u+2: a tile loop ahead while the queue is long,
+//            only after the loop near its end (a wave never holds two waiting units then).
+// With an LPT plan (from_idx / from_pos) n_wg workgroups walk their unit lists instead.
 //
 // Replaces, from the reference: layers/kernels/sparse_attention.cu:2953-3190 (balanced,
 // persistent workgroups over the LPT plan), :2111-2403 (one workgroup per unit) and the
 // dispatcher :3192-3228.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "rt_common.h"
+
 
 namespace {
 
@@ -47,10 +61,11 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
-
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef const int __attribute__((address_space(4))) const_int;   // loads through it are scalar loads
 
 template <typename T> struct Mma;
 template <> struct Mma<_Float16> {
@@ -70,6 +85,19 @@ template <> struct Mma<_Float16> {
     out = __builtin_bit_cast(v8, w);
     return s;
   }
+  // pipelined loop: two values of P rounded to nearest (a value beyond fp16's range must become
+  // infinite: that is how the loop's caller learns that the row outgrew its reference), their sums
+  // kept in packed halves
+  static constexpr bool kPackedSum = true;
+  __device__ static uint32_t two(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
+  }
+  __device__ static uint32_t add(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, a) + __builtin_bit_cast(f16x2, b));
+  }
+  __device__ static float fold(uint32_t a, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), f16x2{1, 1}, acc, false);
+  }
 };
 template <> struct Mma<__bf16> {
   typedef bf16x8 v8;
@@ -83,13 +111,23 @@ template <> struct Mma<__bf16> {
     for (int e = 0; e < 8; ++e) out[e] = static_cast<__bf16>(p[e]);
     return ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
   }
+  static constexpr bool kPackedSum = false;
+  __device__ static uint32_t two(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+  }
+  __device__ static uint32_t add(uint32_t a, uint32_t) { return a; }
+  __device__ static float fold(uint32_t, float acc) { return acc; }
 };
 
-// A row's reference maximum only moves when the 32 values P = 2^(score - reference) a lane holds
-// for one key tile add up to more than 2^11 (no single P can then exceed 2^11, far inside fp16's
-// range, and P keeps its full relative precision at any magnitude): the row sum the kernel needs
-// anyway doubles as the overflow test.
+// Moving-maximum loop: a row's reference maximum only moves when the 32 values P = 2^(score -
+// reference) a lane holds for one key tile add up to more than 2^11 (no single P can then exceed
+// 2^11, far inside fp16's range, and P keeps its full relative precision at any magnitude): the row
+// sum the kernel needs anyway doubles as the overflow test.
 constexpr float SUM_LIMIT = 2048.0f;
+// Pipelined loop: the lane's two queries share one reference; if their own maxima over the first 32
+// keys lie further apart than this (log2 units), the smaller row's P would sink towards fp16's
+// denormals and the unit takes the moving-maximum loop instead.
+constexpr float MAX_REFERENCE_GAP = 8.0f;
 
 // Online-softmax state of one wave for its 64 queries: O^T as [d tile][query tile].
 struct State {
@@ -115,10 +153,10 @@ __device__ inline void load_tile(const T* __restrict__ tile, int lane, typename 
   for (int i = 0; i < 8; ++i) f[i] = *reinterpret_cast<const v8*>(tile + i * 512 + lane * 8);
 }
 
-// Streams key blocks row[first], row[first + step], ... of one (sequence, head) through the
-// state.  kbase / vbase point at block 0 of that (sequence, head); n = blocks in the sequence.
-// The row's block ids are fetched 64 at a time into one register (lane j holds entry j) and
-// handed out with v_readlane: one memory round trip per unit instead of one per key block.
+// Moving-maximum loop.  Streams key blocks row[first], row[first + step], ... of one (sequence,
+// head) through the state.  kbase / vbase point at block 0 of that (sequence, head); n = blocks in
+// the sequence.  The row's block ids are fetched 64 at a time into one register (lane j holds
+// entry j) and handed out with v_readlane: one memory round trip per unit instead of one per key block.
 template <typename T, bool MASKED>
 __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __restrict__ vbase,
                                     const int* __restrict__ row, int first, int step, int cnt, int n, int tail,
@@ -235,48 +273,65 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
   }
 }
 
-// Writes the wave's 64x64 output tile, O^T[d = 32t + 8*(e>>2) + 4*(lane>>5) + (e&3)]
-// [query 32nt + (lane&31)] * w, to out[token][h*64 + d].  The tile is transposed through a
-// wave-private LDS region (64 rows of 64 + 4 elements) so that every global store covers
-// whole 128-byte row segments: 8 lanes x 16 bytes per row.
-constexpr int STAGE_ROW = 68;                       // elements; 136 bytes keeps ds_write_b64 conflict free
-constexpr int STAGE_BYTES = 64 * STAGE_ROW * 2;     // 8704 bytes per wave
+// v_permlane32_swap: the upper 32 lanes of a change places with the lower 32 lanes of b.  Written as
+// assembly: through the builtin, with both operands holding the same value, the compiler used the
+// first result for both.  (s_nop: a vector instruction may just have written the operands.)
+__device__ inline void swap_halves(unsigned& a, unsigned& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+// maximum / sum over lane l and lane l ^ 32, in both lanes
+__device__ inline float pair_max(float x) {
+  unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+  swap_halves(a, b);
+  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+__device__ inline float pair_sum(float x) {
+  unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+  swap_halves(a, b);
+  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+}
 
+// Writes the wave's 64x64 output tile, O^T[d = 32t + 8*(e>>2) + 4*(lane>>5) + (e&3)]
+// [query 32nt + (lane&31)] * w, to out[token][h*64 + d].  A lane holds 4 consecutive d of its query
+// per accumulator quad and its partner lane (lane ^ 32) the next 4: the two swap quads so that every
+// lane stores 16 bytes and the pair 32 consecutive bytes of the token's row.
 template <typename T>
 __device__ inline void store_output(T* __restrict__ out_unit, int64_t row_stride, int lane, const State& st,
-                                    const float (&w)[2], T* __restrict__ stage) {
-  typedef typename Mma<T>::v4 v4;
-  typedef typename Mma<T>::v8 v8;
+                                    const float (&w)[2]) {
   const int l32 = lane & 31, hi = lane >> 5;
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
-    T* sp = stage + (32 * nt + l32) * STAGE_ROW + 4 * hi;
+    T* row = out_unit + int64_t(32 * nt + l32) * row_stride + (hi ? 0 : 8);
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int c4 = 0; c4 < 4; ++c4) {
-        v4 r;
+      for (int c4 = 0; c4 < 4; c4 += 2) {
+        uint32_t x[2], y[2];                                     // quads c4 and c4 + 1, rounded and packed
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r[e] = static_cast<T>(st.o[t][nt][4 * c4 + e] * w[nt]);
-        *reinterpret_cast<v4*>(sp + 32 * t + 8 * c4) = r;
+        for (int j = 0; j < 2; ++j) {
+          x[j] = Mma<T>::two(st.o[t][nt][4 * c4 + 2 * j] * w[nt], st.o[t][nt][4 * c4 + 2 * j + 1] * w[nt]);
+          y[j] = Mma<T>::two(st.o[t][nt][4 * c4 + 4 + 2 * j] * w[nt], st.o[t][nt][4 * c4 + 5 + 2 * j] * w[nt]);
+        }
+        // upper half of y <-> lower half of x: lower lanes end up with quad c4 + 1 of both lanes, upper lanes with quad c4
+        swap_halves(y[0], x[0]);
+        swap_halves(y[1], x[1]);
+        const u32x4 v = {y[0], y[1], x[0], x[1]};
+        *reinterpret_cast<u32x4*>(row + 32 * t + 8 * c4) = v;
       }
   }
-  __builtin_amdgcn_wave_barrier();                  // same wave wrote it: LDS is in order per wave
-  const int r8 = lane >> 3, c8 = (lane & 7) * 8;
-#pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int row = 8 * it + r8;
-    const v4* src = reinterpret_cast<const v4*>(stage + row * STAGE_ROW + c8);   // rows are 8-byte aligned
-    const v4 lo = src[0], up = src[1];
-    const v8 v = {lo[0], lo[1], lo[2], lo[3], up[0], up[1], up[2], up[3]};
-    *reinterpret_cast<v8*>(out_unit + int64_t(row) * row_stride + c8) = v;
-  }
-  __builtin_amdgcn_wave_barrier();
 }
 
 struct Unit {
   int h, i, n, g0;
   int tail;               // tokens in the sequence's last block that are real (64: none padded)
+};
+
+// One unit's row of the to-block CSR, for the wave that runs it (all fields wave-uniform).
+struct Row {
+  Unit u;
+  int p0, cnt;            // the row is to_idx[p0 .. p0 + cnt)
+  int goff;               // byte offset of the unit's (sequence, head) group inside K and V^T
+  int first_off;          // byte offset of the row's first tile inside K and V^T
 };
 
 template <typename T> struct Args {
@@ -288,17 +343,27 @@ template <typename T> struct Args {
   // optional: Q taken from the QKV projection's own output rows [tokens, 3 * heads * 64] (columns
   // 0 .. heads*64-1), bias added and scale applied while loading; q is then unused
   const T* q_rows; const T* q_bias; float q_scale;
+  int* queues;                           // QUEUE_INTS ints of device memory, all zero when the kernel starts
+  int* queues_clear;                     // the counters of a later launch: this launch puts them back to zero
 };
 
 constexpr int MAX_BATCH = 1024;         // sequences per launch (geometry is kept in LDS)
+constexpr int MAX_BLOCKS = 4096;        // 64-token blocks per launch (the row table is kept in LDS)
+constexpr int MAX_HEADS_QROWS = 64;     // heads whose query bias fits the LDS copy
+// Queue counters of one launch: 16 of them (tickets of the 8 global-row queues, then of the 8 unit
+// queues), each alone in a 256-byte line: tickets of one line are served one after the other.
+constexpr int QUEUE_STRIDE = 64;                    // ints between two counters
+constexpr int QUEUE_INTS = 16 * QUEUE_STRIDE;
+constexpr int REDO_SLOTS = 32;          // units a wave may put aside for the moving-maximum loop before it runs them
+constexpr int REDO_ENTRIES = 2048;      // LPT plan: entries per workgroup whose pipelined attempt is tracked
 
-// Geometry of the batch in LDS: sb = prefix blocks, gl / bu = prefix counts of the plan-free
-// launch's global items and bundles (per sequence, times heads).
+// Geometry of the batch in LDS.
 struct Geometry {
-  int sb[MAX_BATCH + 1];
-  int gl[MAX_BATCH + 1];
-  int bu[MAX_BATCH + 1];
-  int tail[MAX_BATCH];                  // real tokens in each sequence's last block (64 without padding)
+  int sb[MAX_BATCH + 1];                // prefix blocks
+  uint32_t rows[MAX_BLOCKS];            // j-th row that is not a global row: sequence << 16 | block inside the sequence
+  uint16_t sparse_seq[MAX_BATCH];       // k-th sequence that has global rows
+  uint8_t tail[MAX_BATCH];              // real tokens in each sequence's last block (64 without padding)
+  int n_rows, n_sparse;
 };
 
 __device__ inline int upper_seq(const int* __restrict__ prefix, int batch, int x) {
@@ -312,70 +377,386 @@ __device__ inline int upper_seq(const int* __restrict__ prefix, int batch, int x
 
 __device__ inline bool is_global_row(const Unit& u) { return u.n >= RT_MIN_SPARSE_BLOCKS && (u.i == 0 || u.i == u.n - 1); }
 
+// ---------------------------------------------------------------------------------------------
+// memory requests of the pipelined loop: raw buffer loads, one resource per array, the tile's
+// byte offset in a scalar register and the fragment's in the instruction's immediate field
+// ---------------------------------------------------------------------------------------------
+template <typename T> struct Buffers {
+  __amdgpu_buffer_rsrc_t k, v, q;
+};
+
 template <typename T>
-__device__ inline void load_q(const Args<T>& a, const Unit& u, int lane, typename Mma<T>::v8 (&qf)[2][4]) {
-  typedef typename Mma<T>::v8 v8;
-  if (a.q_rows) {
-    // fragment (nt, c), lane l = dims 16c + 8(l >> 5) .. +7 of query 32nt + (l & 31): a 16-byte run of
-    // the token's row.  Same arithmetic as the split kernel: (x + bias) * scale in fp32, rounded once.
-    const int64_t ld = int64_t(a.heads) * 192;
-    const T* src = a.q_rows + (int64_t(u.g0 + u.i) * 64 + (lane & 31)) * ld + u.h * 64 + (lane >> 5) * 8;
-    const T* bsrc = a.q_bias + u.h * 64 + (lane >> 5) * 8;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const v8 b = *reinterpret_cast<const v8*>(bsrc + c * 16);
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt) {
-        const v8 x = *reinterpret_cast<const v8*>(src + nt * 32 * ld + c * 16);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) qf[nt][c][e] = static_cast<T>((float(x[e]) + float(b[e])) * a.q_scale);
-      }
-    }
-    return;
-  }
-  const T* qt = a.q + (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n + u.i) * 4096;
-#pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-    for (int c = 0; c < 4; ++c) qf[nt][c] = *reinterpret_cast<const v8*>(qt + (nt * 4 + c) * 512 + lane * 8);
+__device__ inline typename Mma<T>::v8 fetch(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(typename Mma<T>::v8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
 
-// One wave, one unit, all of its key blocks.
-template <typename T, bool MASKED>
-__device__ inline void run_solo(const Args<T>& a, const Unit& u, int lane, T* stage) {
-  typename Mma<T>::v8 qf[2][4];
-  const int row = (a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i;
-  const int p0 = __builtin_amdgcn_readfirstlane(a.to_pos[row]);
-  const int cnt = __builtin_amdgcn_readfirstlane(a.to_pos[row + 1]) - p0;
-  load_q<T>(a, u, lane, qf);
-  const int64_t base = (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n) * 4096;
-  State st;
+// Where a unit's 64x64 query tile lies, as MFMA B fragments: fragment (nt, c) is a buffer load at
+// vector offset voff, scalar offset soff + nt * nt_step + c * c_step.
+struct QPlan { int voff, soff, nt_step, c_step; };
+template <typename T>
+__device__ inline QPlan q_plan(const Args<T>& a, const Unit& u, int lane) {
+  QPlan q;
+  if (a.q_rows) {
+    // raw projection rows: fragment (nt, c), lane l = dims 16c + 8(l >> 5) .. +7 of query 32nt + (l & 31),
+    // a 16-byte run of the token's row
+    const int ld = a.heads * 384;                                   // bytes per token row of [T, 3 * heads * 64]
+    q.voff = (lane & 31) * ld + (lane >> 5) * 16;
+    q.soff = (u.g0 + u.i) * 64 * ld + u.h * 128;
+    q.nt_step = 32 * ld;
+    q.c_step = 32;
+  } else {
+    q.voff = lane * 16;
+    q.soff = (u.g0 * a.heads + u.h * u.n + u.i) * 8192;
+    q.nt_step = 4096;
+    q.c_step = 1024;
+  }
+  return q;
+}
+template <typename T>
+__device__ inline typename Mma<T>::v8 fetch_q(const Buffers<T>& b, const QPlan& q, int k) {   // k = 4 nt + c
+  return fetch<T>(b.q, q.voff, q.soff + (k >> 2) * q.nt_step + (k & 3) * q.c_step);
+}
+template <typename T>
+__device__ inline void request_q(const Args<T>& a, const Buffers<T>& b, const Unit& u, int lane,
+                                 typename Mma<T>::v8 (&qf)[2][4]) {
+  const QPlan q = q_plan<T>(a, u, lane);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) qf[k >> 2][k & 3] = fetch_q<T>(b, q, k);
+}
+
+// (x + bias) * scale in fp32, rounded once: the arithmetic of the split kernel.  qbias = LDS copy of the bias.
+template <typename T>
+__device__ inline void finish_q(const Args<T>& a, const T* qbias, const Unit& u, int lane,
+                                typename Mma<T>::v8 (&qf)[2][4]) {
+  typedef typename Mma<T>::v8 v8;
+  if (!a.q_rows) return;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const v8 bb = *reinterpret_cast<const v8*>(qbias + u.h * 64 + c * 16 + (lane >> 5) * 8);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // pinned in fp32 before the rounding, as in the split kernel: multiply and rounding must not fuse
+        float y = (float(qf[nt][c][e]) + float(bb[e])) * a.q_scale;
+        asm volatile("" : "+v"(y));
+        qf[nt][c][e] = static_cast<T>(y);
+      }
+  }
+}
+
+// lane j: byte offset inside K / V^T of the tile of the row's entry first + j * step (the first 64 of them)
+template <typename T>
+__device__ inline int row_offsets(const Args<T>& a, const Row& r, int first, int step, int lane) {
+  const int e = first + lane * step;
+  int blk = e < r.cnt ? a.to_idx[r.p0 + e] : 0;
+  blk = blk < 0 ? 0 : (blk >= r.u.n ? r.u.n - 1 : blk);
+  return r.goff + blk * 8192;
+}
+
+// CSR row bounds through scalar loads
+template <typename T>
+__device__ inline void describe_bounds(const Args<T>& a, const Unit& u, Row& r) {
+  r.u = u;
+  const int row = __builtin_amdgcn_readfirstlane((a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i);
+  const_int* pos = (const_int*)(uintptr_t)(a.to_pos);
+  r.p0 = pos[row];
+  r.cnt = pos[row + 1] - r.p0;
+  r.goff = (u.g0 * a.heads + u.h * u.n) * 8192;
+}
+// the row's first block, through a scalar load
+template <typename T>
+__device__ inline void describe_first(const Args<T>& a, Row& r) {
+  const_int* idx = (const_int*)(uintptr_t)(a.to_idx);
+  int blk = r.cnt > 0 ? idx[r.p0] : 0;
+  blk = blk < 0 ? 0 : (blk >= r.u.n ? r.u.n - 1 : blk);
+  r.first_off = r.goff + blk * 8192;
+}
+
+// A short row's block ids through scalar loads (they do not queue behind the tile requests, and
+// what they return is not a pending vector load inside the tile loop): 16 entries starting at the
+// row's first.  The caller has checked that p0 + 16 does not pass the end of to_idx.
+constexpr int SHORT_ROW = 16;
+typedef int i32x8 __attribute__((ext_vector_type(8), aligned(4)));
+typedef const i32x8 __attribute__((address_space(4))) const_ids8;
+template <typename T>
+__device__ inline void request_short_row(const Args<T>& a, const Row& r, int (&blk)[SHORT_ROW]) {
+  const_ids8* p = (const_ids8*)(uintptr_t)(a.to_idx + r.p0);
+  const i32x8 lo = p[0], hi = p[1];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) { blk[j] = lo[j]; blk[8 + j] = hi[j]; }
+}
+// lane j (< 16): byte offset inside K / V^T of the tile of the row's entry j
+__device__ inline int short_row_offsets(const Row& r, const int (&blk)[SHORT_ROW], int lane) {
+  int ids = 0;
+#pragma unroll
+  for (int j = 0; j < SHORT_ROW; ++j) {
+    int bj = blk[j];
+    bj = bj < 0 ? 0 : (bj >= r.u.n ? r.u.n - 1 : bj);
+    ids = lane == j ? r.goff + bj * 8192 : ids;
+  }
+  return ids;
+}
+
+#define SB() __builtin_amdgcn_sched_barrier(0)
+
+// The pipelined loop's registers.
+template <typename T> struct Tiles {
+  typename Mma<T>::v8 qf[2][4], kf[8], vf[8];
+};
+
+// first tile of a row, requested in the loop's own order: K's first key half, then the halves the
+// loop's first step does not request itself (so the loop's waits, which count requests still in
+// flight, come out the same on its first trip as on any other)
+template <typename T>
+__device__ inline void request_first(const Buffers<T>& b, int so, int lane, Tiles<T>& t) {
+  const int vo = lane * 16;
+#pragma unroll
+  for (int f = 0; f < 4; ++f) t.kf[f] = fetch<T>(b.k, vo + f * 1024, so);
+  SB();
+#pragma unroll
+  for (int f = 4; f < 8; ++f) t.kf[f] = fetch<T>(b.k, vo + f * 1024, so);
+#pragma unroll
+  for (int f = 0; f < 4; ++f) t.vf[(f & 1) + 4 * (f >> 1)] = fetch<T>(b.v, vo + ((f & 1) + 4 * (f >> 1)) * 1024, so);
+  SB();
+  // the loop's first step multiplies an all-zero P with V^T's second key half, which is only
+  // requested after it: whatever those registers hold must be finite
+#pragma unroll
+  for (int f = 0; f < 4; ++f)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) t.vf[(f & 1) + 2 + 4 * (f >> 1)][e] = static_cast<T>(0.f);
+}
+
+// reference of the pipelined loop: maximum over the row's first 32 keys, shared by the lane's two
+// queries.  False if the two queries' maxima lie too far apart.
+template <typename T>
+__device__ inline bool fast_reference(const Tiles<T>& t, float& mref) {
+  typedef Mma<T> P;
+  f32x16 s0 = {}, s1 = {};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    s0 = P::run(t.kf[c], t.qf[0][c], s0);
+    s1 = P::run(t.kf[c], t.qf[1][c], s1);
+  }
+  float m0 = s0[0], m1 = s1[0];
+#pragma unroll
+  for (int e = 1; e < 16; ++e) { m0 = fmaxf(m0, s0[e]); m1 = fmaxf(m1, s1[e]); }
+  m0 = pair_max(m0);
+  m1 = pair_max(m1);
+  mref = fmaxf(m0, m1);
+  return !__any(!(fabsf(m0 - m1) <= MAX_REFERENCE_GAP));           // false also for NaN / infinite scores
+}
+
+// The pipelined tile loop over `my` (1..64) tiles whose byte offsets sit in the lanes of `ids`; the
+// first tile is in flight or there (request_first).  so_after >= 0: the last tile's steps request that
+// tile (the first one of the wave's next row) instead of a dummy.  next_q(k), k = 0..7: requests
+// fragment k of the next row's queries into t.qf; called in the last tile's last two steps, once
+// the score products have read the fragment it replaces.
+struct NoNextQ { __device__ void operator()(int) const {} };
+template <typename T, typename NextQ>
+__device__ inline void fast_loop(const Buffers<T>& b, int ids, int my, const int& so_after, int lane, float mref,
+                                 Tiles<T>& t, State& st, NextQ next_q) {
+  typedef typename Mma<T>::v8 v8;
+  typedef Mma<T> P;
   state_init(st);
-  stream_tiles<T, MASKED>(a.k + base, a.vt + base, a.to_idx + p0, 0, 1, cnt, u.n, u.tail, lane, qf, st);
+  st.m[0] = st.m[1] = mref;
+  f32x16 negm;                                        // the score products' C operand
+#pragma unroll
+  for (int e = 0; e < 16; ++e) negm[e] = -mref;
+  int vo = lane * 16;
+  auto ldk = [&](int f, int so) { t.kf[f] = fetch<T>(b.k, vo + f * 1024, so); };
+  auto ldv = [&](int f, int so) { t.vf[f] = fetch<T>(b.v, vo + f * 1024, so); };
+  f32x16 sc[2];
+  v8 pb[2][2];
+  float l0 = 0.f, l1 = 0.f;
+  int so_cur = __builtin_amdgcn_readlane(ids, 0);
+  // Everything requested so far must have arrived before the loop is entered (its first step needs
+  // most of it anyway).  The waits inside the loop count the requests in flight; the compiler
+  // derives them from the state at the loop's entry as well as from the loop's own requests, and
+  // anything still pending there turns them into waits for all requests.
+  __builtin_amdgcn_s_waitcnt(0x0F70);                 // vmcnt(0)
+  SB();
+  // pipeline prologue: scores of the first accumulator tile; an all-zero P for the first step's PV slot
+  sc[0] = negm;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) sc[0] = P::run(t.kf[c], t.qf[0][c], sc[0]);
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pb[1][s][e] = static_cast<T>(0.f);
+
+  // one tile: four steps; `last` (a std::bool_constant): the row's last tile
+  auto tile = [&](int so_next, auto last) {
+    constexpr bool LAST = decltype(last)::value;
+    // keeps the fragment offsets inside the loop body, where they fold into the requests' immediate fields
+    asm volatile("" : "+v"(vo));
+#pragma unroll
+    for (int S = 0; S < 4; ++S) {
+      // consume sc[S & 1] (tile a[S]), produce sc[(S + 1) & 1] (a[S + 1]), multiply pb[(S + 1) & 1] (a[S - 1])
+      const int nt = S & 1;
+      const int ktn = ((S + 1) & 3) >> 1, ntn = (S + 1) & 1;          // a[S + 1]
+      const int ktp = ((S + 3) & 3) >> 1, ntp = (S + 3) & 1;          // a[S - 1]
+      f32x16& cur = sc[S & 1];
+      f32x16& nxt = sc[(S + 1) & 1];
+      v8 (&pprev)[2] = pb[(S + 1) & 1];
+      float p[16];
+      uint32_t w[8];
+      uint32_t t01 = 0, t23 = 0, t45 = 0, t67 = 0;
+      float lacc = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        SB();
+        // matrix slot
+        if ((i & 1) == 0) {
+          const int c = i >> 1;
+          // the last tile's last step has no following scores to start: its slots request the next row's queries
+          if (!(LAST && S == 3)) nxt = P::run(t.kf[ktn * 4 + c], t.qf[ntn][c], c == 0 ? negm : nxt);
+        } else {
+          const int tt = (i >> 1) & 1, s = i >> 2;
+          st.o[tt][ntp] = P::run(t.vf[tt * 4 + 2 * ktp + s], pprev[s], st.o[tt][ntp]);
+        }
+        // tile requests: one per slot in the steps whose registers are free
+        if (S == 1) { if (i < 4) ldk(i, so_next); else { const int f = (i & 1) + 2 + 4 * ((i >> 1) & 1); ldv(f, so_cur); } }
+        if (S == 3) { if (i < 4) ldk(4 + i, so_next); else { const int f = (i & 1) + 4 * ((i >> 1) & 1); ldv(f, so_next); } }
+        // the next row's queries: first query half after this row's last use of it (step 1), second after step 2's
+        if (LAST && S == 2 && (i & 1) == 1) next_q(i >> 1);
+        if (LAST && S == 3 && (i & 1) == 0) next_q(4 + (i >> 1));
+        SB();
+        // vector slot: two exponentials, rounding and sums of the previous slot's pair
+        p[2 * i] = __builtin_amdgcn_exp2f(cur[2 * i]);
+        p[2 * i + 1] = __builtin_amdgcn_exp2f(cur[2 * i + 1]);
+        if (i > 0) {
+          w[i - 1] = P::two(p[2 * i - 2], p[2 * i - 1]);
+          if (!P::kPackedSum) lacc += p[2 * i - 2] + p[2 * i - 1];
+        }
+        if (P::kPackedSum) {
+          if (i == 2) t01 = P::add(w[0], w[1]);
+          if (i == 4) t23 = P::add(w[2], w[3]);
+          if (i == 5) t01 = P::add(t01, t23);
+          if (i == 6) t45 = P::add(w[4], w[5]);
+          if (i == 7) t01 = P::add(t01, t45);
+        }
+      }
+      SB();
+      w[7] = P::two(p[14], p[15]);
+      if (P::kPackedSum) {
+        t67 = P::add(w[6], w[7]);
+        t01 = P::add(t01, t67);
+        if (nt == 0) l0 = P::fold(t01, l0); else l1 = P::fold(t01, l1);
+      } else {
+        lacc += p[14] + p[15];
+        if (nt == 0) l0 += lacc; else l1 += lacc;
+      }
+      u32x4 lo = {w[0], w[1], w[2], w[3]}, up = {w[4], w[5], w[6], w[7]};
+      pb[S & 1][0] = __builtin_bit_cast(v8, lo);
+      pb[S & 1][1] = __builtin_bit_cast(v8, up);
+      SB();
+    }
+  };
+
+  for (int e = 0; e + 1 < my; ++e) {
+    const int so_next = __builtin_amdgcn_readlane(ids, (e + 1) & 63);
+    tile(so_next, std::false_type{});
+    so_cur = so_next;
+  }
+  tile(so_after >= 0 ? so_after : so_cur, std::true_type{});
+  // pipeline epilogue: the last tile's a[3] (second key half, second query half)
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) st.o[tt][1] = P::run(t.vf[tt * 4 + 2 + s], pb[1][s], st.o[tt][1]);
+  st.l[0] = l0;
+  st.l[1] = l1;
+}
+
+__device__ inline bool sums_finite(const State& st) { return !__any(!(st.l[0] < INFINITY) || !(st.l[1] < INFINITY)); }
+
+// moving-maximum loop on entries first, first + step, ... of row r
+template <typename T, bool MASKED>
+__device__ inline void slow_row(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Row& r, int first, int step,
+                                int lane, bool have_q, typename Mma<T>::v8 (&qf)[2][4], State& st) {
+  if (!have_q) {
+    request_q<T>(a, b, r.u, lane, qf);
+    finish_q<T>(a, qbias, r.u, lane, qf);
+  }
+  state_init(st);
+  const int64_t gbase = int64_t(r.goff >> 1);
+  stream_tiles<T, MASKED>(a.k + gbase, a.vt + gbase, a.to_idx + r.p0, first, step, r.cnt, r.u.n, r.u.tail, lane, qf, st);
+}
+
+// Entries first, first + step, ... of row r through the state with the pipelined loop, no hand-over
+// from or to another row.  False: the row has to be run with the moving-maximum loop instead (more
+// than 64 entries for this wave, or scores that outgrew the reference); the state is then undefined.
+template <typename T>
+__device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Row& r, int first, int step,
+                                int lane, State& st) {
+  Tiles<T> t;
+  state_init(st);
+  first = __builtin_amdgcn_readfirstlane(first);
+  const int my = __builtin_amdgcn_readfirstlane((r.cnt - first + step - 1) / step);     // this wave's entries
+  if (my <= 0) return true;
+  if (my > 64) return false;
+  const int ids = row_offsets<T>(a, r, first, step, lane);
+  request_q<T>(a, b, r.u, lane, t.qf);
+  request_first<T>(b, __builtin_amdgcn_readlane(ids, 0), lane, t);
+  finish_q<T>(a, qbias, r.u, lane, t.qf);
+  float mref;
+  if (!fast_reference<T>(t, mref)) return false;
+  fast_loop<T>(b, ids, my, -1, lane, mref, t, st, NoNextQ{});
+  return sums_finite(st);
+}
+
+// normalises the state and writes the unit's output tile
+template <typename T>
+__device__ inline void finish_unit(const Args<T>& a, const Unit& u, int lane, State& st) {
   float w[2];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
-    const float l = st.l[nt] + __shfl_xor(st.l[nt], 32, 64);
-    w[nt] = 1.0f / fmaxf(l, 1e-30f);
-  }
+  for (int nt = 0; nt < 2; ++nt) w[nt] = __builtin_amdgcn_rcpf(fmaxf(pair_sum(st.l[nt]), 1e-30f));
   const int64_t stride = int64_t(a.heads) * 64;
-  store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w, stage);
+  store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w);
 }
 
-// Four waves, one unit: wave w streams key blocks w, w+4, ...; tree merge through LDS.
-template <typename T, bool MASKED>
-__device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int wave, float* park) {
-  typename Mma<T>::v8 qf[2][4];
-  const int row = (a.plan_heads > 1 ? u.h : 0) * a.nb_total + u.g0 + u.i;
-  const int p0 = __builtin_amdgcn_readfirstlane(a.to_pos[row]);
-  const int cnt = __builtin_amdgcn_readfirstlane(a.to_pos[row + 1]) - p0;
-  load_q<T>(a, u, lane, qf);
-  const int64_t base = (int64_t(u.g0) * a.heads + int64_t(u.h) * u.n) * 4096;
+template <typename T>
+__device__ inline Row describe(const Args<T>& a, const Unit& u) {
+  Row r;
+  describe_bounds<T>(a, u, r);
+  describe_first<T>(a, r);
+  return r;
+}
+
+// One wave, one unit, all of its key blocks.  FAST: pipelined loop; false = the unit has to be run
+// again with FAST = false (nothing was written).
+template <typename T, bool MASKED, bool FAST>
+__device__ inline bool run_solo(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Unit& u, int lane) {
+  const Row r = describe<T>(a, u);
   State st;
-  state_init(st);
-  stream_tiles<T, MASKED>(a.k + base, a.vt + base, a.to_idx + p0, wave, 4, cnt, u.n, u.tail, lane, qf, st);
+  if (FAST) {
+    if (!fast_row<T>(a, b, qbias, r, 0, 1, lane, st)) return false;
+  } else {
+    typename Mma<T>::v8 qf[2][4];
+    slow_row<T, MASKED>(a, b, qbias, r, 0, 1, lane, false, qf, st);
+  }
+  finish_unit<T>(a, u, lane, st);
+  return true;
+}
+
+// Four waves, one unit: wave w streams key blocks w, w+4, ...; tree merge through LDS.  FAST:
+// pipelined loop; false (the same in all four waves) = the unit has to be run again with FAST = false.
+template <typename T, bool MASKED, bool FAST>
+__device__ inline bool run_split4(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Unit& u, int lane,
+                                  int wave, float* park) {
+  const Row r = describe<T>(a, u);
+  State st;
+  if (FAST) {
+    const bool ok = fast_row<T>(a, b, qbias, r, wave, 4, lane, st);
+    if (__syncthreads_or(!ok)) return false;          // also: the park is free (previous item is over)
+  } else {
+    typename Mma<T>::v8 qf[2][4];
+    slow_row<T, MASKED>(a, b, qbias, r, wave, 4, lane, false, qf, st);
+    __syncthreads();                                  // the park is free (previous item is over)
+  }
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) st.l[nt] += __shfl_xor(st.l[nt], 32, 64);
+  for (int nt = 0; nt < 2; ++nt) st.l[nt] = pair_sum(st.l[nt]);
 
   auto dump = [&](float* slot) {
 #pragma unroll
@@ -405,7 +786,6 @@ __device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int
           st.o[t][nt][e] = st.o[t][nt][e] * a0 + slot[((t * 2 + nt) * 16 + e) * 64 + lane] * a1;
     }
   };
-  __syncthreads();                                    // the park is free (previous item is over)
   if (wave >= 2) dump(park + (wave - 2) * (68 * 64));
   __syncthreads();
   if (wave < 2) absorb(park + wave * (68 * 64));
@@ -416,41 +796,43 @@ __device__ inline void run_split4(const Args<T>& a, const Unit& u, int lane, int
     absorb(park);
     float w[2];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) w[nt] = 1.0f / fmaxf(st.l[nt], 1e-30f);
+    for (int nt = 0; nt < 2; ++nt) w[nt] = __builtin_amdgcn_rcpf(fmaxf(st.l[nt], 1e-30f));
     const int64_t stride = int64_t(a.heads) * 64;
-    // slot 1 of the park was consumed before the third barrier: reuse it as the staging tile
-    store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w,
-                    reinterpret_cast<T*>(park + 68 * 64));
+    store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w);
   }
-  __syncthreads();                                    // the park is free again (solo waves stage their output in it)
+  return true;
 }
 
-__device__ __host__ inline int bundles_per_head(int n) {
-  return n >= RT_MIN_SPARSE_BLOCKS ? (n - 2 + 3) / 4 : (n + 3) / 4;
+// One ticket of a queue counter, in lane 0: a request, not yet waited for.  A buffer atomic whose
+// resource covers just the counter: every lane executes it, lanes 1..63 address past the end and
+// are dropped by the hardware, so no branch (and no wait at the end of one) surrounds the request.
+__device__ inline __amdgpu_buffer_rsrc_t ticket_counter(int* p) { return __builtin_amdgcn_make_buffer_rsrc(p, 0, 4, 0x00020000); }
+__device__ inline int request_ticket(__amdgpu_buffer_rsrc_t counter, int lane) {
+  return __builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, counter, lane * 4, 0, 1);
+}
+// the same instruction; if `really` (wave-uniform) is false all lanes address past the end: nothing is drawn
+__device__ inline int request_ticket_if(__amdgpu_buffer_rsrc_t counter, int lane, bool really) {
+  return __builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, counter, lane * 4 + (really ? 0 : 4), 0, 1);
 }
 
 // Persistent workgroups (two per CU).
-//
-// With an LPT plan (from_idx / from_pos): workgroup c walks its slice of the plan; global rows
-// are shared by its four waves, runs of up to four other units go one per wave.
-//
-// Without a plan the kernel makes its own schedule.  Two kinds of items:
-//   global item : one global row (first or last block of a sequence of >= 12 blocks), 4 waves
-//   bundle      : up to 4 consecutive other rows of one (sequence, head), one per wave
-// numbered sequence-major, then head.  Workgroups are dealt to the 8 XCDs round-robin by the
-// hardware; the workgroups of XCD x share the x-th eighth of the global items FIRST (they are
-// the long ones) and then the x-th eighth of the bundles, which covers (nearly) the same
-// (sequence, head) groups, so a group's K/V tiles stay in one L2.
 template <typename T, bool MASKED>
 __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
-  // 34816 bytes: two parked wave states for the global-row merge, or four output staging tiles
+  // 34816 bytes: two parked wave states for the global-row merge
   __shared__ __attribute__((aligned(16))) float park[2 * 68 * 64];
   __shared__ Geometry geo;
-  static_assert(4 * STAGE_BYTES <= sizeof(float) * 2 * 68 * 64, "staging tiles must fit in the park");
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  T* stage = reinterpret_cast<T*>(reinterpret_cast<char*>(park) + wave * STAGE_BYTES);
+  __shared__ __attribute__((aligned(16))) T qbias[MAX_HEADS_QROWS * 64];
+  __shared__ int s_item;
+  __shared__ int redo[4][REDO_SLOTS];                 // per wave: units put aside for the moving-maximum loop
+  __shared__ int redo_rows[REDO_SLOTS];               // per workgroup: global rows put aside
+  __shared__ uint8_t s_redo[REDO_ENTRIES];            // LPT plan: entries of the workgroup's slice to run again
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
+  // geometry: prefix blocks, the list of rows that are not global rows, the sequences that have global rows
+  int* const row_base = reinterpret_cast<int*>(park);            // per sequence: rows listed before it (scratch use of the park)
   for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
+  if (a.q_rows)
+    for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias[i] = a.q_bias[i];
   __syncthreads();
   for (int i = threadIdx.x; i < a.batch; i += 256) {
     int t = 64;
@@ -458,21 +840,40 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       t = a.seq_tokens[i] - 64 * (geo.sb[i + 1] - geo.sb[i] - 1);
       t = t < 1 ? 1 : (t > 64 ? 64 : t);
     }
-    geo.tail[i] = t;
+    geo.tail[i] = uint8_t(t);
   }
   if (threadIdx.x == 0) {
-    int g = 0, b = 0;
+    int rows = 0, sparse = 0;
     for (int s = 0; s < a.batch; ++s) {
-      geo.gl[s] = g;
-      geo.bu[s] = b;
+      row_base[s] = rows;
       const int n = geo.sb[s + 1] - geo.sb[s];
-      g += (n >= RT_MIN_SPARSE_BLOCKS ? 2 : 0) * a.heads;
-      b += bundles_per_head(n) * a.heads;
+      if (n >= RT_MIN_SPARSE_BLOCKS) {
+        geo.sparse_seq[sparse++] = uint16_t(s);
+        rows += n - 2;
+      } else {
+        rows += n;
+      }
     }
-    geo.gl[a.batch] = g;
-    geo.bu[a.batch] = b;
+    geo.n_rows = rows;
+    geo.n_sparse = sparse;
   }
   __syncthreads();
+  for (int g = threadIdx.x; g < a.nb_total; g += 256) {
+    const int s = upper_seq(geo.sb, a.batch, g);
+    const int n = geo.sb[s + 1] - geo.sb[s], i = g - geo.sb[s];
+    const bool sparse = n >= RT_MIN_SPARSE_BLOCKS;
+    if (!sparse || (i > 0 && i < n - 1)) geo.rows[row_base[s] + i - (sparse ? 1 : 0)] = uint32_t(s) << 16 | uint32_t(i);
+  }
+  __syncthreads();
+
+  Buffers<T> b;
+  {
+    const uint32_t kv_bytes = uint32_t(a.nb_total) * uint32_t(a.heads) * 8192u;
+    b.k = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a.k), 0, kv_bytes, 0x00020000);
+    b.v = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a.vt), 0, kv_bytes, 0x00020000);
+    b.q = a.q_rows ? __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a.q_rows), 0, kv_bytes * 3u, 0x00020000)
+                   : __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a.q), 0, kv_bytes, 0x00020000);
+  }
 
   auto unit_of_flat = [&](int unit) {               // flat id = blk + head * n_s + seq_start * heads
     int lo = 0, hi = a.batch;
@@ -491,60 +892,231 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
   };
 
   if (a.from_pos) {
-    int p = a.from_pos[blockIdx.x];
-    const int end = a.from_pos[blockIdx.x + 1];
+    // LPT plan: global rows are shared by the workgroup's four waves, runs of up to four other units go
+    // one per wave.  Two passes over the workgroup's slice: the pipelined loop first, then, for what
+    // it handed back (s_redo: one flag per plan entry of the slice, at most REDO_ENTRIES), the
+    // moving-maximum loop.
+    const int begin = a.from_pos[blockIdx.x], end = a.from_pos[blockIdx.x + 1];
     const int n_units = a.nb_total * a.heads;
-    while (p < end) {
-      // the next four plan entries in one round trip
-      const int mine_id = (p + wave < end) ? a.from_idx[p + wave] : -1;
-      int ids4[4];
+    auto walk = [&](auto fast) {
+      constexpr bool FAST = decltype(fast)::value;
+      int p = begin;
+      while (p < end) {
+        // the next four plan entries in one round trip
+        const int mine_id = (p + wave < end) ? a.from_idx[p + wave] : -1;
+        int ids4[4];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) ids4[w] = (p + w < end) ? a.from_idx[p + w] : -1;
-      if (ids4[0] < 0 || ids4[0] >= n_units) { ++p; continue; }
-      const Unit first = unit_of_flat(ids4[0]);
-      if (is_global_row(first)) {
-        run_split4<T, MASKED>(a, first, lane, wave, park);
-        ++p;
-        continue;
+        for (int w = 0; w < 4; ++w) ids4[w] = (p + w < end) ? a.from_idx[p + w] : -1;
+        if (ids4[0] < 0 || ids4[0] >= n_units) { ++p; continue; }
+        const Unit first = unit_of_flat(ids4[0]);
+        const bool tracked = p - begin < REDO_ENTRIES;         // entries past the flags take the moving-maximum loop
+        if (is_global_row(first)) {
+          const bool todo = FAST ? (!MASKED && tracked) : (MASKED || !tracked || s_redo[p - begin] != 0);
+          if (todo) {
+            const bool ok = run_split4<T, MASKED, FAST>(a, b, qbias, first, lane, wave, park);
+            if (FAST && threadIdx.x == 0) s_redo[p - begin] = ok ? 0 : 1;
+          }
+          ++p;
+          continue;
+        }
+        int run = 1;
+        while (run < 4 && ids4[run] >= 0 && ids4[run] < n_units && !is_global_row(unit_of_flat(ids4[run]))) ++run;
+        if (wave < run) {
+          const int e = p + wave - begin;
+          const bool trk = e < REDO_ENTRIES;
+          const bool todo = FAST ? (!MASKED && trk) : (MASKED || !trk || s_redo[e] != 0);
+          if (todo) {
+            const bool ok = run_solo<T, MASKED, FAST>(a, b, qbias, unit_of_flat(mine_id), lane);
+            if (FAST && lane == 0) s_redo[e] = ok ? 0 : 1;
+          }
+        }
+        p += run;
       }
-      int run = 1;
-      while (run < 4 && ids4[run] >= 0 && ids4[run] < n_units && !is_global_row(unit_of_flat(ids4[run]))) ++run;
-      if (wave < run) run_solo<T, MASKED>(a, unit_of_flat(mine_id), lane, stage);
-      p += run;
-    }
+    };
+    walk(std::true_type{});
+    __syncthreads();
+    walk(std::false_type{});
     return;
   }
 
-  const int n_glob = geo.gl[a.batch], n_bund = geo.bu[a.batch];
-  const int x = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
-  const int g_lo = int(int64_t(n_glob) * x / 8), g_cnt = int(int64_t(n_glob) * (x + 1) / 8) - g_lo;
-  const int b_lo = int(int64_t(n_bund) * x / 8), b_cnt = int(int64_t(n_bund) * (x + 1) / 8) - b_lo;
-  for (int k = blockIdx.x >> 3; k < g_cnt + b_cnt; k += per_xcd) {
-    Unit u;
-    if (k < g_cnt) {
-      const int item = g_lo + k;
-      const int s = upper_seq(geo.gl, a.batch, item);
-      const int rem = item - geo.gl[s];
+  const int xcd = blockIdx.x & 7;
+  const __amdgpu_buffer_rsrc_t gq = ticket_counter(a.queues + xcd * QUEUE_STRIDE);          // this XCD's global-row queue
+  const __amdgpu_buffer_rsrc_t uq = ticket_counter(a.queues + (8 + xcd) * QUEUE_STRIDE);    // this XCD's unit queue
+  if (blockIdx.x == 0 && threadIdx.x < 16) a.queues_clear[threadIdx.x * QUEUE_STRIDE] = 0;
+
+  // phase 1: global rows, one per workgroup.  A pair = the first and the last row of one (sequence,
+  // head): both stream the same K / V^T tiles, so they are consecutive tickets of the same XCD.
+  // Pairs are numbered head-major and XCD x owns the x-th eighth of them: the same heads whose
+  // other rows it runs in phase 2.
+  {
+    const int n_pairs = geo.n_sparse * a.heads;
+    const int p_lo = int(int64_t(n_pairs) * xcd / 8), p_hi = int(int64_t(n_pairs) * (xcd + 1) / 8);
+    const int n_glob = 2 * (p_hi - p_lo);             // tickets of this XCD that are rows
+    auto unit_of_row = [&](int ticket) {
+      const int pair = p_lo + (ticket >> 1);
+      const int h = pair / geo.n_sparse;
+      const int s = geo.sparse_seq[pair - h * geo.n_sparse];
+      Unit u;
       u.g0 = geo.sb[s];
       u.n = geo.sb[s + 1] - u.g0;
       u.tail = geo.tail[s];
-      u.h = rem >> 1;
-      u.i = (rem & 1) ? u.n - 1 : 0;
-      run_split4<T, MASKED>(a, u, lane, wave, park);
-      continue;
+      u.h = h;
+      u.i = (ticket & 1) ? u.n - 1 : 0;
+      return u;
+    };
+    bool drained = false;
+    while (!drained) {
+      int n_rows_redo = 0;
+      while (n_rows_redo < REDO_SLOTS) {
+        if (wave == 0) {
+          const int k = __builtin_amdgcn_readfirstlane(request_ticket(gq, lane));
+          if (lane == 0) s_item = k;
+        }
+        __syncthreads();
+        const int item = s_item;
+        __syncthreads();
+        if (item >= n_glob) { drained = true; break; }
+        bool ok = false;
+        if (!MASKED) ok = run_split4<T, MASKED, true>(a, b, qbias, unit_of_row(item), lane, wave, park);
+        if (!ok) {
+          if (threadIdx.x == 0) redo_rows[n_rows_redo] = item;
+          ++n_rows_redo;
+        }
+      }
+      __syncthreads();
+      for (int r = 0; r < n_rows_redo; ++r)
+        run_split4<T, MASKED, false>(a, b, qbias, unit_of_row(redo_rows[r]), lane, wave, park);
+      __syncthreads();
     }
-    const int item = b_lo + (k - g_cnt);
-    const int s = upper_seq(geo.bu, a.batch, item);
-    const int rem = item - geo.bu[s];
-    u.g0 = geo.sb[s];
-    u.n = geo.sb[s + 1] - u.g0;
-    u.tail = geo.tail[s];
-    const int per_head = bundles_per_head(u.n);
-    u.h = rem / per_head;
-    const int bundle = rem - u.h * per_head;
-    const bool sparse = u.n >= RT_MIN_SPARSE_BLOCKS;
-    u.i = (sparse ? 1 : 0) + 4 * bundle + wave;
-    if (u.i <= (sparse ? u.n - 2 : u.n - 1)) run_solo<T, MASKED>(a, u, lane, stage);
+  }
+
+  // phase 2: all other rows; every wave draws single units.  Item = head * n_rows + j (j-th listed
+  // row), XCD x owns the x-th eighth of the items.
+  {
+    const int lane_id = lane;
+    const int n_rows = geo.n_rows;
+    const int total = n_rows * a.heads;
+    const int lo = int(int64_t(total) * xcd / 8), hi = int(int64_t(total) * (xcd + 1) / 8);
+    const float inv_rows = 1.0f / float(n_rows > 0 ? n_rows : 1);
+    auto unit_of = [&](int item) {
+      int h = int((float(item) + 0.5f) * inv_rows);
+      int j = item - h * n_rows;
+      if (j < 0) { --h; j += n_rows; }
+      if (j >= n_rows) { ++h; j -= n_rows; }
+      const uint32_t e = geo.rows[j];
+      const int s = int(e >> 16);
+      Unit u;
+      u.g0 = geo.sb[s];
+      u.n = geo.sb[s + 1] - u.g0;
+      u.tail = geo.tail[s];
+      u.h = h;
+      u.i = int(e & 0xffffu);
+      return u;
+    };
+    auto item_of = [&](int ticket) {                  // -1: the queue is drained
+      const int k = __builtin_amdgcn_readfirstlane(ticket);
+      return lo + k < hi ? lo + k : -1;
+    };
+    const_int* pos_all = (const_int*)(uintptr_t)(a.to_pos);
+    const int idx_total = pos_all[a.plan_heads * a.nb_total];       // entries in to_idx
+    const int waves_per_xcd = int(gridDim.x >> 3) * 4;
+    int n_redo = 0;
+    int item = item_of(request_ticket(uq, lane));
+    int item_nx = item >= 0 ? item_of(request_ticket(uq, lane)) : -1;
+    while (item >= 0 || n_redo > 0) {
+      // pipelined loop on one unit after the other, each handing the next one its first tile.  A wave
+      // holds the unit it runs and the next one; the one after that is drawn when the tile loop ends.
+      if (item >= 0) {
+        Tiles<T> t;
+        Row cur;
+        int blk[SHORT_ROW];
+        describe_bounds<T>(a, unit_of(item), cur);
+        bool cur_short = cur.cnt >= 1 && cur.cnt <= SHORT_ROW && cur.p0 + SHORT_ROW <= idx_total;
+        int ids = 0;
+        cur.first_off = 0;
+        if (cur_short) {
+          request_short_row<T>(a, cur, blk);
+          ids = short_row_offsets(cur, blk, lane_id);
+          cur.first_off = __builtin_amdgcn_readlane(ids, 0);
+        }
+        bool primed = false;
+        while (item >= 0 && n_redo < REDO_SLOTS) {
+          // what the code below derives from the lane number is derived again for every unit, not
+          // kept in registers across the tile loop
+          int lane = lane_id;
+          asm volatile("" : "+v"(lane));
+          const bool has_next = item_nx >= 0;
+          Row nx = cur;
+          if (has_next) describe_bounds<T>(a, unit_of(item_nx), nx);        // scalar loads, waited for below
+          State st;
+          bool ok = !MASKED && cur_short;
+          if (ok && !primed) {
+            request_q<T>(a, b, cur.u, lane, t.qf);
+            request_first<T>(b, cur.first_off, lane, t);
+          }
+          float mref = 0.f;
+          if (ok) {
+            finish_q<T>(a, qbias, cur.u, lane, t.qf);
+            ok = fast_reference<T>(t, mref);
+          }
+          // the next row's block ids: requested here, looked at in the loop's last tile
+          bool nx_short = false;
+          nx.first_off = -1;
+          if (has_next) {
+            nx_short = nx.cnt >= 1 && nx.cnt <= SHORT_ROW && nx.p0 + SHORT_ROW <= idx_total;
+            if (nx_short) {
+              request_short_row<T>(a, nx, blk);
+              int b0 = blk[0];
+              b0 = b0 < 0 ? 0 : (b0 >= nx.u.n ? nx.u.n - 1 : b0);
+              nx.first_off = nx.goff + b0 * 8192;
+            }
+          }
+          // The unit after the next one.  Far from the end of the queue its ticket is drawn here, a
+          // whole tile loop before it is looked at; near the end only after the loop, so that a wave
+          // never sits on two waiting units while others run dry.  Both requests are always issued
+          // (one of them addresses nothing): no branch, so the waits further down count requests.
+          const bool far = has_next && hi - item_nx > 2 * waves_per_xcd;
+          const int t_early = request_ticket_if(uq, lane, far);
+          int item_after = -1;
+          primed = false;
+          if (ok) {
+            const QPlan qn = q_plan<T>(a, nx.u, lane);      // without a next unit: this unit's queries again
+            fast_loop<T>(b, ids, cur.cnt, nx.first_off, lane, mref, t, st,
+                         [&](int k) { t.qf[k >> 2][k & 3] = fetch_q<T>(b, qn, k); });
+            lane = lane_id;
+            asm volatile("" : "+v"(lane));
+            const int t_late = request_ticket_if(uq, lane, has_next && !far);
+            SB();
+            primed = nx_short;
+            if (sums_finite(st)) {
+              finish_unit<T>(a, cur.u, lane, st);
+              SB();
+              item_after = has_next ? item_of(far ? t_early : t_late) : -1;
+            } else {
+              if (lane == 0) redo[wave][n_redo] = item;
+              ++n_redo;
+              item_after = has_next ? item_of(far ? t_early : t_late) : -1;
+            }
+          } else {
+            if (lane == 0) redo[wave][n_redo] = item;
+            ++n_redo;
+            const int t_late = request_ticket_if(uq, lane, has_next && !far);
+            item_after = has_next ? item_of(far ? t_early : t_late) : -1;
+          }
+          item = item_nx;
+          item_nx = item_after;
+          cur = nx;
+          cur_short = nx_short;
+          if (nx_short) ids = short_row_offsets(nx, blk, lane);
+        }
+      }
+      // the units put aside: moving-maximum loop
+      for (int r = 0; r < n_redo; ++r) {
+        const int it = __builtin_amdgcn_readfirstlane(redo[wave][r]);
+        run_solo<T, MASKED, false>(a, b, qbias, unit_of(it), lane_id);
+      }
+      n_redo = 0;
+    }
   }
 }
 
@@ -560,6 +1132,27 @@ unsigned plan_free_workgroups() {
   return cached;
 }
 
+// Queue counters of the library's own launches: a ring of slots, so that launches which overlap on
+// different streams do not share counters.  A launch leaves its slot used; launch i clears the slot
+// that launch i + QUEUE_SLOTS / 2 will take.
+constexpr int QUEUE_SLOTS = 64;
+int* library_queues(int* err, int** clear) {
+  static int* base[64] = {};
+  static unsigned next[64] = {};
+  int dev = 0;
+  *err = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { *err = 1; return nullptr; }
+  if (!base[dev]) {
+    int* p = nullptr;
+    if (hipMalloc(&p, sizeof(int) * QUEUE_INTS * QUEUE_SLOTS) != hipSuccess) { *err = 2; return nullptr; }
+    if (hipMemset(p, 0, sizeof(int) * QUEUE_INTS * QUEUE_SLOTS) != hipSuccess) { *err = 3; return nullptr; }
+    base[dev] = p;
+  }
+  const unsigned slot = next[dev]++ % QUEUE_SLOTS;
+  *clear = base[dev] + ((slot + QUEUE_SLOTS / 2) % QUEUE_SLOTS) * QUEUE_INTS;
+  return base[dev] + slot * QUEUE_INTS;
+}
+
 }  // namespace
 
 namespace {
@@ -573,31 +1166,41 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
              batch, total_blocks, heads);
   RT_REQUIRE(plan_heads == 1 || plan_heads == heads, RT_EINVAL, "plan_heads=%d must be 1 or heads=%d", plan_heads, heads);
   RT_REQUIRE((from_idx == nullptr) == (from_pos == nullptr), RT_EINVAL, "from_idx and from_pos go together");
-  RT_REQUIRE(int64_t(total_blocks) * heads < (int64_t(1) << 31), RT_EINVAL, "too many units");
+  RT_REQUIRE(int64_t(total_blocks) * heads * 8192 * 3 < (int64_t(1) << 31), RT_EINVAL,
+             "batch too large: %d blocks x %d heads (byte offsets are 32-bit)", total_blocks, heads);
   RT_REQUIRE(batch <= MAX_BATCH, RT_EINVAL, "at most %d sequences per launch, got %d", MAX_BATCH, batch);
+  RT_REQUIRE(total_blocks <= MAX_BLOCKS, RT_EINVAL, "at most %d blocks (%d tokens) per launch, got %d blocks", MAX_BLOCKS,
+             MAX_BLOCKS * 64, total_blocks);
+  RT_REQUIRE(!q_rows || heads <= MAX_HEADS_QROWS, RT_EINVAL, "queries from the projection rows: at most %d heads, got %d",
+             MAX_HEADS_QROWS, heads);
   RT_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(q_rows) | reinterpret_cast<uintptr_t>(q_bias) |
                reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(vt) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0,
              RT_EINVAL, "q (or qkv and its bias), k, vt, out must be 16-byte aligned");
   if (dtype == RT_F32) return rt::fail(RT_ENOSYS, "block-sparse attention runs in fp16 or bf16 (fp32 accumulation)");
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16, RT_EINVAL, "unknown dtype %d", dtype);
   unsigned grid;
+  int* queues = nullptr;
+  int* queues_clear = nullptr;
   if (from_idx) {
     RT_REQUIRE(n_wg >= 1, RT_EINVAL, "balanced launch needs n_wg >= 1, got %d", n_wg);
     grid = unsigned(n_wg);
   } else {
     grid = plan_free_workgroups();
+    int err = 0;
+    queues = library_queues(&err, &queues_clear);
+    if (!queues) return rt::fail(RT_ENOMEM, "no device memory for the work queues (step %d)", err);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == RT_F16) {
     Args<_Float16> a{(const _Float16*)q, (const _Float16*)k, (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch,
                      heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
-                     (const _Float16*)q_rows, (const _Float16*)q_bias, q_scale};
+                     (const _Float16*)q_rows, (const _Float16*)q_bias, q_scale, queues, queues_clear};
     if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<_Float16, true>), dim3(grid), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((bs_attention_kernel<_Float16, false>), dim3(grid), dim3(256), 0, st, a);
   } else {
     Args<__bf16> a{(const __bf16*)q, (const __bf16*)k, (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads,
                    total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
-                   (const __bf16*)q_rows, (const __bf16*)q_bias, q_scale};
+                   (const __bf16*)q_rows, (const __bf16*)q_bias, q_scale, queues, queues_clear};
     if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<__bf16, true>), dim3(grid), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((bs_attention_kernel<__bf16, false>), dim3(grid), dim3(256), 0, st, a);
   }

@@ -472,7 +472,14 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
     const int dst = ((4 * (row >> 5) + (col8 >> 1)) * 64 + (row & 31) + 32 * (col8 & 1)) * 8 + (col & 7);
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      if (WITH_Q) x[0][i] = (x[0][i] + b[0][i]) * q_scale;
+      if (WITH_Q) {
+        // The product is pinned in fp32 before it is rounded to the output type: left alone the
+        // compiler may fuse multiply and rounding into one instruction that rounds once, and
+        // the attention kernel's own copy of this arithmetic must give the same bits.
+        float y = (x[0][i] + b[0][i]) * q_scale;
+        asm volatile("" : "+v"(y));
+        x[0][i] = y;
+      }
       x[1][i] = x[1][i] + b[1][i];
       vtile[row][col + i] = x[2][i] + b[2][i];
     }
