@@ -163,6 +163,26 @@ int rt_bs_attention_fwd_qrows(const void* qkv, const void* qkv_bias, float q_sca
                               const int* from_idx, const int* from_pos, int n_wg, int dtype,
                               void* stream);
 
+/* rt_bs_attention_fwd_masked for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  The other attention entry points take the kernel's queue counters from a ring that the
+ * library allocates on a device's first launch; this one keeps them in a static device array of
+ * RT_NO_ALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends, and calls
+ * no hipMalloc, hipFree or other allocating routine.  It always runs the kernel's own enumeration (no
+ * from_idx/from_pos plan; that launch uses no counters and allocates nothing in any entry point).
+ * Limits: batch <= RT_NO_ALLOC_MAX_BATCH and total_blocks <= RT_NO_ALLOC_MAX_BLOCKS, else RT_EINVAL.
+ * Every call on one GPU uses the same counters, cleared by a small kernel ahead of the launch: calls
+ * that overlap on one GPU (two streams, two threads) race and give wrong results; calls on one stream,
+ * or otherwise ordered, are fine.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress): make that call outside a graph capture. */
+#define RT_NO_ALLOC_SCRATCH_BYTES 8192
+#define RT_NO_ALLOC_MAX_BATCH 1024
+#define RT_NO_ALLOC_MAX_BLOCKS 4096
+int rt_bs_attention_fwd_no_alloc(const void* q, const void* k, const void* vt, void* out,
+                                 const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
+                                 int total_blocks, int heads, const int* to_idx, const int* to_pos,
+                                 int plan_heads, int dtype, void* stream);
+
 /* Replaces kernels::add_bias_and_layernorm_kernel (layers/kernels/
  * add_bias_and_layernorm.cu:268-285): out = LN(out + bias + residual) * gamma + beta,
  * in place on out[rows, hidden]; hidden a multiple of 8. */

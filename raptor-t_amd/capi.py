@@ -23,7 +23,7 @@ EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
-    "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows",
+    "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows", "rt_bs_attention_fwd_no_alloc",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm_set_retuning", "rt_gemm",
     "rt_gemm_bias_act", "rt_gemm_bt", "rt_sequence_pool", "rt_pooler_dense_tanh",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
@@ -62,6 +62,7 @@ def lib():
         L.rt_bs_attention_fwd.argtypes = [vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
         L.rt_bs_attention_fwd_masked.argtypes = [vp, vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
         L.rt_bs_attention_fwd_qrows.argtypes = [vp, vp, F, vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
+        L.rt_bs_attention_fwd_no_alloc.argtypes = [vp, vp, vp, vp, vp, vp, I, I, I, vp, vp, I, I, vp]
         L.rt_bias_residual_layernorm.argtypes = [vp, vp, vp, vp, vp, L64, I, F, I, vp]
         L.rt_bias_gelu.argtypes = [vp, vp, L64, I, I, vp]
         L.rt_gemm_create.argtypes = [ctypes.POINTER(vp)]
@@ -204,6 +205,17 @@ def bs_attention_fwd(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_
     check(lib().rt_bs_attention_fwd_masked(_dp(q), _dp(k), _dp(vt), _dp(out), _dp(seq_blocks_dev), _dp(seq_tokens_dev),
                                            batch, nb, heads, _dp(to_idx), _dp(to_pos), plan_heads, _dp(from_idx),
                                            _dp(from_pos), n_wg, _dtype_code(out), _stream()))
+
+
+def bs_attention_fwd_no_alloc(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads, seq_tokens_dev=None):
+    """bs_attention_fwd through the entry point that allocates no device memory (static queue counters)."""
+    batch = seq_blocks_dev.numel() - 1
+    nb = out.shape[0] // 64
+    if seq_tokens_dev is not None and seq_tokens_dev.numel() != batch:
+        raise ValueError("seq_tokens_dev needs one entry per sequence")
+    check(lib().rt_bs_attention_fwd_no_alloc(_dp(q), _dp(k), _dp(vt), _dp(out), _dp(seq_blocks_dev), _dp(seq_tokens_dev),
+                                             batch, nb, heads, _dp(to_idx), _dp(to_pos), plan_heads, _dtype_code(out),
+                                             _stream()))
 
 
 def bs_attention_fwd_qrows(qkv, qkv_bias, q_scale, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads,

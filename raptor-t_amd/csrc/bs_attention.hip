@@ -49,6 +49,7 @@
 // dispatcher :3192-3228.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "rt_common.h"
@@ -1139,9 +1140,11 @@ constexpr int QUEUE_SLOTS = 64;
 int* library_queues(int* err, int** clear) {
   static int* base[64] = {};
   static unsigned next[64] = {};
+  static std::mutex mu;
   int dev = 0;
   *err = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { *err = 1; return nullptr; }
+  std::lock_guard<std::mutex> lock(mu);
   if (!base[dev]) {
     int* p = nullptr;
     if (hipMalloc(&p, sizeof(int) * QUEUE_INTS * QUEUE_SLOTS) != hipSuccess) { *err = 2; return nullptr; }
@@ -1160,7 +1163,8 @@ namespace {
 int launch_attention(const void* q, const void* q_rows, const void* q_bias, float q_scale, const void* k, const void* vt,
                      void* out, const int* seq_blocks_dev, const int* seq_tokens_dev, int batch, int total_blocks,
                      int heads, const int* to_idx, const int* to_pos, int plan_heads, const int* from_idx,
-                     const int* from_pos, int n_wg, int dtype, void* stream) {
+                     const int* from_pos, int n_wg, int dtype, void* stream, int* own_queues = nullptr,
+                     int* own_queues_clear = nullptr) {
   RT_REQUIRE((q || (q_rows && q_bias)) && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1, RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d",
              batch, total_blocks, heads);
@@ -1186,9 +1190,14 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
     grid = unsigned(n_wg);
   } else {
     grid = plan_free_workgroups();
-    int err = 0;
-    queues = library_queues(&err, &queues_clear);
-    if (!queues) return rt::fail(RT_ENOMEM, "no device memory for the work queues (step %d)", err);
+    if (own_queues) {
+      queues = own_queues;
+      queues_clear = own_queues_clear;
+    } else {
+      int err = 0;
+      queues = library_queues(&err, &queues_clear);
+      if (!queues) return rt::fail(RT_ENOMEM, "no device memory for the work queues (step %d)", err);
+    }
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == RT_F16) {
@@ -1237,4 +1246,51 @@ extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt,
                                    void* stream) {
   return rt_bs_attention_fwd_masked(q, k, vt, out, seq_blocks_dev, nullptr, batch, total_blocks, heads, to_idx, to_pos,
                                     plan_heads, from_idx, from_pos, n_wg, dtype, stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------------
+// Its queue counters live in this array instead of the library's allocated ring.  First half: the
+// counters of the running launch, zeroed by a fill kernel ahead of every launch; second half: where
+// that launch's own clearing store goes (nobody reads it).  In host code the array's name is only a
+// stand-in: its address on a device comes from hipGetSymbolAddress, once per device.
+constexpr int NO_ALLOC_SCRATCH_INTS = 2 * QUEUE_INTS;
+static_assert(NO_ALLOC_SCRATCH_INTS * sizeof(int) == RT_NO_ALLOC_SCRATCH_BYTES, "header and kernel disagree on the scratch size");
+static_assert(RT_NO_ALLOC_MAX_BATCH <= MAX_BATCH && RT_NO_ALLOC_MAX_BLOCKS <= MAX_BLOCKS, "header limits exceed the kernel's");
+static __device__ __align__(256) int scratch[NO_ALLOC_SCRATCH_INTS];
+
+namespace {
+
+__global__ void clear_queue_counters(int* counters) { counters[threadIdx.x * QUEUE_STRIDE] = 0; }
+
+int* no_alloc_scratch() {
+  static int* ptr[64] = {};
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+    ptr[dev] = static_cast<int*>(p);
+  }
+  return ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int rt_bs_attention_fwd_no_alloc(const void* q, const void* k, const void* vt, void* out,
+                                            const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
+                                            int total_blocks, int heads, const int* to_idx, const int* to_pos,
+                                            int plan_heads, int dtype, void* stream) {
+  RT_REQUIRE(q, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(batch >= 1 && batch <= RT_NO_ALLOC_MAX_BATCH && total_blocks >= batch && total_blocks <= RT_NO_ALLOC_MAX_BLOCKS,
+             RT_EINVAL, "rt_bs_attention_fwd_no_alloc takes at most %d sequences and %d blocks (%d tokens), got %d and %d",
+             RT_NO_ALLOC_MAX_BATCH, RT_NO_ALLOC_MAX_BLOCKS, RT_NO_ALLOC_MAX_BLOCKS * 64, batch, total_blocks);
+  int* counters = no_alloc_scratch();
+  if (!counters) return rt::fail(RT_EIO, "the address of the static scratch array is not available on this device");
+  hipLaunchKernelGGL(clear_queue_counters, dim3(1), dim3(QUEUE_INTS / QUEUE_STRIDE), 0, static_cast<hipStream_t>(stream), counters);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return rt::fail(RT_EIO, "clearing the queue counters failed: %s", hipGetErrorString(e));
+  return launch_attention(q, nullptr, nullptr, 1.0f, k, vt, out, seq_blocks_dev, seq_tokens_dev, batch, total_blocks, heads,
+                          to_idx, to_pos, plan_heads, nullptr, nullptr, 0, dtype, stream, counters, counters + QUEUE_INTS);
 }
