@@ -55,31 +55,139 @@ def hbm_roofline(name, bytes_per_launch, us_per_launch, traffic=None):
             "us_per_launch": us_per_launch}
 
 
+def host_cores():
+    """Threads the CPU baselines run on: every core this job may use.  That is the scheduler affinity of the
+    process, further limited by OMP_NUM_THREADS when the host sets it (a GPU box shares its cores between the
+    jobs of its GPUs and exports its share there); os.cpu_count() is printed beside it."""
+    n = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    if env.isdigit() and int(env) >= 1:
+        n = min(n, int(env))
+    return max(n, 1)
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def timed_median(fn, warmup, reps, budget_s):
+    """Median seconds of fn(); stops early, after at least three timed runs, once `budget_s` is used up."""
+    for _ in range(warmup):
+        fn()
+    times, t_start = [], time.perf_counter()
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+        if len(times) >= 3 and time.perf_counter() - t_start > budget_s:
+            break
+    return float(np.median(times)), len(times)
+
+
+def cpu_baseline_config1():
+    """Benchmark config 1 itself on the host cores: ONE BigBird-base encoder layer, batch 1, 1024 tokens, hidden
+    768, 12 x 64 heads, FFN 3072, block 64, 2 global + 3 window + 3 random blocks, fp32, N(0, 0.02) weights,
+    N(0, 1) input, seed 0; the oracle's layer (PyTorch CPU), on every core of the job and on one thread."""
+    from oracle import layer as ol
+    from oracle import metadata as md
+    hidden, heads, ffn, lens = 768, 12, 3072, [1024]
+    g = torch.Generator().manual_seed(0)
+    w = ol.random_layer_weights(hidden, ffn, g)
+    x = torch.randn(sum(lens), hidden, generator=g)
+    sb = md.seq_prefix_blocks(lens)
+    idx, pos = md.hf_to_index(lens, 0, heads)
+    fn = lambda: ol.encoder_layer(x, w, heads, sb, idx, pos, heads)
+    cores = host_cores()
+    before = torch.get_num_threads()
+    torch.set_num_threads(cores)
+    t_all, n_all = timed_median(fn, 3, 20, 8.0)
+    torch.set_num_threads(1)
+    t_one, n_one = timed_median(fn, 1, 20, 8.0)
+    torch.set_num_threads(before)
+    return {"value": sum(lens) / t_all, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "ms_per_layer": t_all * 1e3,
+            "sample": "benchmark config 1 itself: one BigBird-base layer, batch 1 x 1024 tokens, fp32, the oracle's layer "
+                      "(torch CPU); median of %d runs on %d threads" % (n_all, cores),
+            "one_thread": {"value": sum(lens) / t_one, "unit": "tokens/s", "cores": 1, "ms_per_layer": t_one * 1e3,
+                           "runs": n_one},
+            "host_cpu_count": os.cpu_count(), "cpu_model": cpu_model()}
+
+
 def cpu_baseline_layer(seq_lens, hidden, heads, ffn, layers, sample_seqs, reps=3):
     """Oracle encoder layer (PyTorch-CPU fp32, the reference oracle's algorithm) on the first
     `sample_seqs` sequences of the batch, scaled by tokens to the whole batch and by the layer
-    count to the whole encoder."""
+    count to the whole encoder: the GPU line's own workload and unit, on every core of the job."""
     from oracle import layer as ol
     from oracle import metadata as md
-    cores = min(os.cpu_count() or 1, 16)
+    cores = host_cores()
     torch.set_num_threads(cores)
     lens = list(seq_lens[:sample_seqs])
     g = torch.Generator().manual_seed(0)
     w = ol.random_layer_weights(hidden, ffn, g)
     x = torch.randn(sum(lens), hidden, generator=g)
     sb = md.seq_prefix_blocks(lens)
-    idx, pos = md.hf_to_index(lens, 0, heads)
-    times = []
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        ol.encoder_layer(x, w, heads, sb, idx, pos, heads)
-        times.append(time.perf_counter() - t0)
-    t_layer = float(np.median(times))
+    idx, pos = md.hf_to_index(lens, 0, heads, max_pos=max(4096, max(lens)))
+    t_layer, n = timed_median(lambda: ol.encoder_layer(x, w, heads, sb, idx, pos, heads), 0, reps, 12.0)
     t_batch = t_layer * (sum(seq_lens) / sum(lens)) * layers
     return {"value": len(seq_lens) / t_batch, "unit": "seqs/s", "cores": cores, "kind": "port",
             "sample": "oracle encoder layer (torch CPU fp32) on the first %d sequences (%d tokens), median of %d, "
                       "scaled by tokens to the batch and x%d layers; %.2f s per sampled layer"
-                      % (len(lens), sum(lens), reps, layers, t_layer)}
+                      % (len(lens), sum(lens), n, layers, t_layer)}
+
+
+def cpu_baseline(seq_lens, hidden, heads, ffn, layers, sample_seqs):
+    """The CPU figures of one encoder line: config 1 as it stands (all cores and one thread), and under
+    `this_workload` the line's own workload from a bounded sample, in the line's unit."""
+    out = cpu_baseline_config1()
+    out["this_workload"] = cpu_baseline_layer(seq_lens, hidden, heads, ffn, layers, sample_seqs)
+    return out
+
+
+def cpu_baseline_attention(steps=20):
+    """CPU-side figure of the isolated-attention line: the oracle's block-sparse attention on ONE of the eight
+    sequences (4096 tokens, 12 heads, fp32), in algorithmic GFLOP/s, every core of the job."""
+    from oracle import attention as oa
+    from oracle import metadata as md
+    heads, lens = 12, [4096]
+    cores = host_cores()
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(lens[0], heads, 64, generator=g) for _ in range(3))
+    sb = md.seq_prefix_blocks(lens)
+    idx, pos = md.hf_to_index(lens, 0, heads)
+    t_one, n = timed_median(lambda: oa.csr_attention(q, k, v, sb, idx, pos, heads), 1, steps, 15.0)
+    flops = block_pairs(list(sb), heads) * PAIR_FLOP
+    return {"value": flops / t_one / 1e9, "unit": "GFLOP/s", "cores": cores, "kind": "port", "ms": t_one * 1e3,
+            "ms_scaled_to_batch_8": 8 * t_one * 1e3,
+            "sample": "oracle block-sparse attention (torch CPU fp32) on one sequence of 4096 tokens, 12 heads; "
+                      "median of %d" % n, "host_cpu_count": os.cpu_count(), "cpu_model": cpu_model()}
+
+
+def cpu_baseline_membound(steps=20):
+    """CPU-side figure of the memory-bound sweep's smallest point (8192 tokens, fp32): the oracle's
+    bias + residual + LayerNorm over [8192, 768] and bias + GELU over [8192, 3072], in algorithmic GB/s."""
+    from oracle import layer as ol
+    cores = host_cores()
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    t = 8192
+    x, r = torch.randn(t, 768, generator=g), torch.randn(t, 768, generator=g)
+    b, ga, be = (torch.randn(768, generator=g) for _ in range(3))
+    t_ln, _ = timed_median(lambda: ol.bias_residual_layernorm(x, r, b, ga, be, 1e-5), 3, steps, 5.0)
+    y, b2 = torch.randn(t, 3072, generator=g), torch.randn(3072, generator=g)
+    t_gelu, _ = timed_median(lambda: ol.bias_gelu(y, b2), 3, steps, 5.0)
+    return {"value": 3 * t * 768 * 4 / t_ln / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "oracle bias + residual + LayerNorm (torch CPU fp32) over [8192, 768], 3 tensor passes of 4 bytes",
+            "gelu": {"value": 2 * t * 3072 * 4 / t_gelu / 1e9, "unit": "GB/s",
+                     "sample": "oracle bias + GELU over [8192, 3072], 2 tensor passes of 4 bytes"},
+            "host_cpu_count": os.cpu_count(), "cpu_model": cpu_model()}
 
 
 def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos=4096):
@@ -128,6 +236,8 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
         step()
     timing_all = mb.cxx.timing_collect()
     meta.terminate_thread()
+    # outside the timed region: a step that produced a NaN or an Inf anywhere is not a measurement
+    assert bool(torch.isfinite(hidden_states).all()), "the encoder's output is not finite"
 
     ms_step = elapsed / args.steps * 1e3
     per = {k: v[0] / v[1] for k, v in timing_all.items() if v[1]}
@@ -174,7 +284,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
                          "steps with every launcher bracketed",
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_layer(seq_lens, hidden, heads, ffn, layers, args.cpu_sample_seqs)
+        out["cpu_baseline"] = cpu_baseline(seq_lens, hidden, heads, ffn, layers, args.cpu_sample_seqs)
     return out
 
 
@@ -221,15 +331,19 @@ def run_attention_only(args):
     else:
         fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads)
     us = time_kernel(fn, args.steps, args.warmup)
+    assert bool(torch.isfinite(out).all()), "the attention output is not finite"
     pairs = block_pairs(sb.tolist(), heads)
     ach = pairs * PAIR_FLOP / (us * 1e-6)
-    return {"metric": "isolated block-sparse attention, batch 8 x 4096, 12 heads x 64, fp16", "value": ach / 1e12,
+    res = {"metric": "isolated block-sparse attention, batch 8 x 4096, 12 heads x 64, fp16", "value": ach / 1e12,
             "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": us / 1e3,
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": "c2 isolated attention", "block_pairs": pairs, "block_limit": args.block_limit,
                        "balanced": args.lpt_plan},
             "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12, "peak": 2500.0,
                          "unit": "TFLOP/s", "frac": ach / 2.5e15, "traffic": None}}
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_attention()
+    return res
 
 
 def run_membound_sweep(args):
@@ -257,11 +371,16 @@ def run_membound_sweep(args):
             e = torch.empty(t, 768, dtype=dt, device="cuda")
             us = time_kernel(lambda: capi.embed_layernorm(ids, pids, tids, word, pos, typ, ga32, be32, e), args.steps, args.warmup)
             rows.append(dict(hbm_roofline("embed_layernorm_kernel", t * 768 * (4 + 2), us), tokens=t, dtype=name, us=us))
+            for nm, buf in (("LayerNorm", x), ("GELU", y), ("embedding", e)):
+                assert bool(torch.isfinite(buf).all()), "%s output at %d tokens is not finite" % (nm, t)
     best_ln = max(r["frac"] for r in rows if r["kernel"].startswith("bias_residual"))
-    return {"metric": "fused add-bias+LayerNorm / bias+GELU achieved HBM GB/s", "value": best_ln * 8000.0, "unit": "GB/s",
+    res = {"metric": "fused add-bias+LayerNorm / bias+GELU achieved HBM GB/s", "value": best_ln * 8000.0, "unit": "GB/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "f16/bf16", "data": "synthetic",
             "config": {"workload": "c4 memory-bound op sweep"}, "sweep": rows}
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline_membound()
+    return res
 
 
 def run_streaming(args):
@@ -311,6 +430,7 @@ def run_streaming(args):
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     meta.terminate_thread()
+    assert bool(torch.isfinite(hs[:sum(batches[-1])]).all()), "the encoder's output is not finite"
     tokens = sum(sum(b) for b in batches[args.warmup:])
     return {"metric": METRIC, "value": 16 * args.steps / elapsed, "unit": "seqs/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True,

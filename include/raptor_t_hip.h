@@ -106,6 +106,13 @@ int rt_meta_block_costs(const int* seq_blocks, int batch, int* out_costs, int64_
 int rt_meta_partition_lpt(const int* seq_blocks, int batch, int heads, int n_wg,
                           int* out_pos, int* out_ids);
 
+/* Host-side check of a work plan before it is handed to a balanced attention launch (no counterpart in
+ * the reference, whose kernel trusts python/util.py:11-34): from_pos[n_wg+1] runs from 0 to
+ * total_blocks*heads without decreasing and from_idx lists every unit id exactly once.  RT_EINVAL otherwise.
+ * The attention kernel itself skips an id outside the range (its rows stay unwritten) rather than fault;
+ * a caller that builds plans of its own calls this first. */
+int rt_meta_check_partition(const int* from_pos, const int* from_idx, int n_wg, int total_blocks, int heads);
+
 /* --------------------------------------------------------------------- GPU kernels */
 
 /* Replaces kernels::add_bias_and_transpose_kernel (layers/kernels/

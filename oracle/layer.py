@@ -58,24 +58,35 @@ def qkv_bias_split(qkv, bias, heads, scale=None):
     return q, k, v
 
 
-def attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block=64):
+def _stored(x, store_dtype):
+    """A tensor as it reads back after a kernel has written it to memory in `store_dtype` (None: kept in fp32).
+    The reference keeps every tensor between two kernels in the model's dtype (fp16: python/modeling_bert.py:63,
+    the buffers of layers/multi_headed_attention.cpp:154-216), so its arithmetic sees these roundings too."""
+    return x if store_dtype is None else x.to(store_dtype).float()
+
+
+def attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block=64, store_dtype=None):
     """QKV projection -> split -> block-sparse attention -> out-proj -> bias+residual+LN
     (layers/multi_headed_attention.cpp:154-216)."""
-    qkv = hidden.float() @ w["qkv_weight"].float()
-    q, k, v = qkv_bias_split(qkv, w["qkv_bias"], heads)
-    ctx = attention.csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block, scale=1.0)
-    proj = ctx @ w["attn_out_weight"].float()
-    return bias_residual_layernorm(proj, hidden, w["attn_out_bias"], w["attn_ln_weight"],
-                                   w["attn_ln_bias"], eps)
+    st = lambda x: _stored(x, store_dtype)
+    qkv = st(hidden.float() @ w["qkv_weight"].float())
+    q, k, v = (st(x) for x in qkv_bias_split(qkv, w["qkv_bias"], heads))
+    ctx = st(attention.csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block, scale=1.0))
+    t = ctx.shape[0]
+    proj = st(ctx.reshape(t, -1) @ w["attn_out_weight"].float())
+    return st(bias_residual_layernorm(proj, hidden, w["attn_out_bias"], w["attn_ln_weight"],
+                                      w["attn_ln_bias"], eps))
 
 
-def encoder_layer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps=1e-5, block=64):
+def encoder_layer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps=1e-5, block=64, store_dtype=None):
     """One layer: attention sub-layer, FFN up + GELU, FFN down + bias+residual+LN with the
-    attention output as the residual (python/modeling_bert.py:172-210)."""
-    attn = attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block)
-    inter = bias_gelu(attn @ w["inter_weight"].float(), w["inter_bias"])
-    out = inter @ w["out_weight"].float()
-    return bias_residual_layernorm(out, attn, w["out_bias"], w["out_ln_weight"], w["out_ln_bias"], eps)
+    attention output as the residual (python/modeling_bert.py:172-210).  store_dtype: the dtype every tensor
+    that passes from one kernel to the next is rounded to (None: all fp32, the plain mathematical layer)."""
+    st = lambda x: _stored(x, store_dtype)
+    attn = attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block, store_dtype)
+    inter = st(bias_gelu(attn @ w["inter_weight"].float(), w["inter_bias"]))
+    out = st(inter @ w["out_weight"].float())
+    return st(bias_residual_layernorm(out, attn, w["out_bias"], w["out_ln_weight"], w["out_ln_bias"], eps))
 
 
 def random_layer_weights(hidden, ffn, generator, std=0.02, dtype=torch.float32):

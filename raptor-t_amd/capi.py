@@ -22,7 +22,7 @@ RT_GEMM_TUNE_ALL = -1
 EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
-    "rt_meta_partition_lpt", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
+    "rt_meta_partition_lpt", "rt_meta_check_partition", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows", "rt_bs_attention_fwd_no_alloc",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm_set_retuning", "rt_gemm",
     "rt_gemm_bias_act", "rt_gemm_bt", "rt_sequence_pool", "rt_pooler_dense_tanh",
@@ -57,6 +57,7 @@ def lib():
         L.rt_meta_build_to_index.argtypes = [i32p, I, I, I, U, I, I, i32p, i32p, L64, i32p, L64]
         L.rt_meta_block_costs.argtypes = [i32p, I, i32p, i64p]
         L.rt_meta_partition_lpt.argtypes = [i32p, I, I, I, i32p, i32p]
+        L.rt_meta_check_partition.argtypes = [i32p, i32p, I, I, I]
         L.rt_qkv_bias_split.argtypes = [vp, vp, vp, vp, vp, vp, I, I, I, F, I, vp]
         L.rt_unpack_head_tiles.argtypes = [vp, vp, vp, I, I, I, I, I, vp]
         L.rt_bs_attention_fwd.argtypes = [vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
@@ -155,6 +156,14 @@ def partition_lpt(seq_blocks, heads, n_wg):
     return pos, ids
 
 
+def check_partition(from_pos, from_idx, total_blocks, heads):
+    """Raises RaptorError unless (from_pos, from_idx) is a work plan that lists every unit exactly once."""
+    pos, ids = _i32(from_pos), _i32(from_idx)
+    if len(ids) != total_blocks * heads or len(pos) < 2:
+        raise ValueError("from_idx needs total_blocks * heads entries and from_pos at least two")
+    check(lib().rt_meta_check_partition(_p(pos), _p(ids), len(pos) - 1, total_blocks, heads))
+
+
 # ------------------------------------------------------------------------------- GPU kernels
 def _dtype_code(t):
     import torch
@@ -166,22 +175,67 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def _dp(t):
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+def _dp(t, dtype=None, numel=None, name="tensor"):
+    """Device pointer of `t` for a kernel argument (None -> NULL).  The kernels dereference it as it is, so a
+    host tensor, a strided view, another dtype or too few elements is refused here: on the GPU each of these
+    would be a memory fault, not an error code."""
+    if t is None:
+        return ctypes.c_void_p(0)
+    if not t.is_cuda:
+        raise ValueError("%s must be a GPU tensor, got one on %s" % (name, t.device))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError("%s must have dtype %s, got %s" % (name, dtype, t.dtype))
+    if numel is not None and t.numel() < numel:
+        raise ValueError("%s holds %d elements, the launch reads %d" % (name, t.numel(), numel))
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _ip(t, numel=None, name="index tensor"):
+    """Device pointer of an int32 index tensor."""
+    import torch
+    return _dp(t, torch.int32, numel, name)
+
+
+def _attention_args(out, k, vt, seq_blocks_dev, heads, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev):
+    """Shapes every attention entry point shares; returns (batch, blocks, n_wg)."""
+    batch = seq_blocks_dev.numel() - 1
+    if out.dim() != 2 or out.shape[0] % 64 or out.shape[1] != heads * 64:
+        raise ValueError("out must be [tokens (a multiple of 64), heads * 64]")
+    nb = out.shape[0] // 64
+    n_wg = 0 if from_pos is None else from_pos.numel() - 1
+    if (from_idx is None) != (from_pos is None):
+        raise ValueError("from_idx and from_pos go together")
+    if plan_heads not in (1, heads):
+        raise ValueError("plan_heads must be 1 or heads")
+    if seq_tokens_dev is not None and seq_tokens_dev.numel() != batch:
+        raise ValueError("seq_tokens_dev needs one entry per sequence")
+    _dp(k, out.dtype, out.numel(), "k"), _dp(vt, out.dtype, out.numel(), "vt"), _dp(out, name="out")
+    _ip(seq_blocks_dev, name="seq_blocks_dev"), _ip(seq_tokens_dev, name="seq_tokens_dev")
+    _ip(to_idx, name="to_idx"), _ip(to_pos, plan_heads * nb + 1, "to_pos")
+    _ip(from_idx, nb * heads, "from_idx"), _ip(from_pos, name="from_pos")
+    return batch, nb, n_wg
 
 
 def qkv_bias_split(qkv, bias, q, k, vt, seq_blocks_dev, heads, q_scale):
     """q may be None: Q is not written (for bs_attention_fwd_qrows)."""
     batch = seq_blocks_dev.numel() - 1
+    if qkv.dim() != 2 or qkv.shape[0] % 64 or qkv.shape[1] != 3 * heads * 64:
+        raise ValueError("qkv must be [tokens (a multiple of 64), 3 * heads * 64]")
     nb = qkv.shape[0] // 64
-    check(lib().rt_qkv_bias_split(_dp(qkv), _dp(bias), _dp(q), _dp(k), _dp(vt), _dp(seq_blocks_dev), batch, nb,
-                                  heads, q_scale, _dtype_code(qkv), _stream()))
+    per = qkv.shape[0] * heads * 64
+    dt = qkv.dtype
+    check(lib().rt_qkv_bias_split(_dp(qkv, name="qkv"), _dp(bias, dt, 3 * heads * 64, "bias"), _dp(q, dt, per, "q"),
+                                  _dp(k, dt, per, "k"), _dp(vt, dt, per, "vt"), _ip(seq_blocks_dev, name="seq_blocks_dev"),
+                                  batch, nb, heads, q_scale, _dtype_code(qkv), _stream()))
 
 
 def unpack_head_tiles(packed, dst, seq_blocks_dev, heads, transposed):
     batch = seq_blocks_dev.numel() - 1
     nb = dst.shape[0] // 64
-    check(lib().rt_unpack_head_tiles(_dp(packed), _dp(dst), _dp(seq_blocks_dev), batch, nb, heads,
+    check(lib().rt_unpack_head_tiles(_dp(packed, dst.dtype, dst.numel(), "packed"), _dp(dst, name="dst"),
+                                     _ip(seq_blocks_dev, name="seq_blocks_dev"), batch, nb, heads,
                                      1 if transposed else 0, _dtype_code(dst), _stream()))
 
 
@@ -192,16 +246,14 @@ Q_SCALE = LOG2E / 8.0          # log2(e) / sqrt(64): what rt_bs_attention_fwd ex
 def bs_attention_fwd(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads,
                      from_idx=None, from_pos=None, seq_tokens_dev=None):
     """seq_tokens_dev: optional int32 device tensor, true token count per sequence (padded tail)."""
-    batch = seq_blocks_dev.numel() - 1
-    nb = out.shape[0] // 64
-    n_wg = 0 if from_pos is None else from_pos.numel() - 1
+    batch, nb, n_wg = _attention_args(out, k, vt, seq_blocks_dev, heads, to_idx, to_pos, plan_heads, from_idx, from_pos,
+                                      seq_tokens_dev)
+    _dp(q, out.dtype, out.numel(), "q")
     if seq_tokens_dev is None:
         check(lib().rt_bs_attention_fwd(_dp(q), _dp(k), _dp(vt), _dp(out), _dp(seq_blocks_dev), batch, nb, heads,
                                         _dp(to_idx), _dp(to_pos), plan_heads, _dp(from_idx), _dp(from_pos), n_wg,
                                         _dtype_code(out), _stream()))
         return
-    if seq_tokens_dev.numel() != batch:
-        raise ValueError("seq_tokens_dev needs one entry per sequence")
     check(lib().rt_bs_attention_fwd_masked(_dp(q), _dp(k), _dp(vt), _dp(out), _dp(seq_blocks_dev), _dp(seq_tokens_dev),
                                            batch, nb, heads, _dp(to_idx), _dp(to_pos), plan_heads, _dp(from_idx),
                                            _dp(from_pos), n_wg, _dtype_code(out), _stream()))
@@ -209,10 +261,8 @@ def bs_attention_fwd(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_
 
 def bs_attention_fwd_no_alloc(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads, seq_tokens_dev=None):
     """bs_attention_fwd through the entry point that allocates no device memory (static queue counters)."""
-    batch = seq_blocks_dev.numel() - 1
-    nb = out.shape[0] // 64
-    if seq_tokens_dev is not None and seq_tokens_dev.numel() != batch:
-        raise ValueError("seq_tokens_dev needs one entry per sequence")
+    batch, nb, _ = _attention_args(out, k, vt, seq_blocks_dev, heads, to_idx, to_pos, plan_heads, None, None, seq_tokens_dev)
+    _dp(q, out.dtype, out.numel(), "q")
     check(lib().rt_bs_attention_fwd_no_alloc(_dp(q), _dp(k), _dp(vt), _dp(out), _dp(seq_blocks_dev), _dp(seq_tokens_dev),
                                              batch, nb, heads, _dp(to_idx), _dp(to_pos), plan_heads, _dtype_code(out),
                                              _stream()))
@@ -221,11 +271,9 @@ def bs_attention_fwd_no_alloc(q, k, vt, out, seq_blocks_dev, heads, to_idx, to_p
 def bs_attention_fwd_qrows(qkv, qkv_bias, q_scale, k, vt, out, seq_blocks_dev, heads, to_idx, to_pos, plan_heads,
                            from_idx=None, from_pos=None, seq_tokens_dev=None):
     """bs_attention_fwd with the queries taken from the [T, 3*H*64] projection output `qkv` (+ qkv_bias, * q_scale)."""
-    batch = seq_blocks_dev.numel() - 1
-    nb = out.shape[0] // 64
-    n_wg = 0 if from_pos is None else from_pos.numel() - 1
-    if seq_tokens_dev is not None and seq_tokens_dev.numel() != batch:
-        raise ValueError("seq_tokens_dev needs one entry per sequence")
+    batch, nb, n_wg = _attention_args(out, k, vt, seq_blocks_dev, heads, to_idx, to_pos, plan_heads, from_idx, from_pos,
+                                      seq_tokens_dev)
+    _dp(qkv, out.dtype, 3 * out.numel(), "qkv"), _dp(qkv_bias, out.dtype, 3 * heads * 64, "qkv_bias")
     if qkv.shape[0] != out.shape[0] or qkv.shape[1] != 3 * heads * 64 or \
             (qkv_bias is not None and qkv_bias.numel() != 3 * heads * 64):
         raise ValueError("qkv must be [tokens, 3 * heads * 64] with a bias of the same width")
@@ -236,13 +284,18 @@ def bs_attention_fwd_qrows(qkv, qkv_bias, q_scale, k, vt, out, seq_blocks_dev, h
 
 def bias_residual_layernorm(out, residual, bias, gamma, beta, eps):
     rows, hidden = out.shape
+    dt = out.dtype
+    _dp(out, name="out"), _dp(residual, dt, out.numel(), "residual")
+    for name, t in (("bias", bias), ("gamma", gamma), ("beta", beta)):
+        _dp(t, dt, hidden, name)
     check(lib().rt_bias_residual_layernorm(_dp(out), _dp(residual), _dp(bias), _dp(gamma), _dp(beta), rows, hidden,
                                            eps, _dtype_code(out), _stream()))
 
 
 def bias_gelu(out, bias):
     rows, width = out.shape
-    check(lib().rt_bias_gelu(_dp(out), _dp(bias), rows, width, _dtype_code(out), _stream()))
+    check(lib().rt_bias_gelu(_dp(out, name="out"), _dp(bias, out.dtype, width, "bias"), rows, width, _dtype_code(out),
+                             _stream()))
 
 
 RT_POOL_FIRST, RT_POOL_LAST, RT_POOL_MEAN, RT_POOL_MAX = 0, 1, 2, 3
@@ -255,7 +308,8 @@ def sequence_pool(hidden, seq_blocks_dev, mode, out, seq_tokens_dev=None):
         raise ValueError("out must be [sequences, width] in the dtype of hidden")
     if seq_tokens_dev is not None and seq_tokens_dev.numel() != batch:
         raise ValueError("seq_tokens_dev needs one entry per sequence")
-    check(lib().rt_sequence_pool(_dp(hidden), _dp(seq_blocks_dev), _dp(seq_tokens_dev), batch, hidden.shape[1], mode,
+    check(lib().rt_sequence_pool(_dp(hidden, name="hidden"), _ip(seq_blocks_dev, name="seq_blocks_dev"),
+                                 _ip(seq_tokens_dev, name="seq_tokens_dev"), batch, hidden.shape[1], mode,
                                  _dp(out), _dtype_code(hidden), _stream()))
     return out
 
@@ -266,6 +320,8 @@ def pooler_dense_tanh(pooled, weight_t, bias, out):
     d_out = weight_t.shape[0]
     if weight_t.shape[1] != d_in or bias.numel() != d_out or tuple(out.shape) != (batch, d_out):
         raise ValueError("shape mismatch")
+    for name, t in (("weight_t", weight_t), ("bias", bias), ("out", out)):
+        _dp(t, pooled.dtype, None, name)
     check(lib().rt_pooler_dense_tanh(_dp(pooled), _dp(weight_t), _dp(bias), _dp(out), batch, d_in, d_out,
                                      _dtype_code(pooled), _stream()))
     return out
@@ -303,9 +359,14 @@ class Gemm:
         """How many of a kind's best solutions the first call with a new M times (0 / 1: none)."""
         check(lib().rt_gemm_set_retuning(self._h, candidates))
 
+    @staticmethod
+    def _operands(a, b, c, m, n, k, bias=None):
+        _dp(a, name="a"), _dp(b, a.dtype, k * n, "b"), _dp(c, a.dtype, m * n, "c"), _dp(bias, a.dtype, n, "bias")
+
     def __call__(self, a, b, c):
         m, k = a.shape
         n = b.shape[1]
+        self._operands(a, b, c, m, n, k)
         check(lib().rt_gemm(self._h, _dp(a), _dp(b), _dp(c), m, n, k, _dtype_code(a), _stream()))
         return c
 
@@ -313,6 +374,7 @@ class Gemm:
         """c = a @ b + bias, through the tanh GELU when epilogue is RT_EPILOGUE_BIAS_GELU, in one kernel."""
         m, k = a.shape
         n = b.shape[1]
+        self._operands(a, b, c, m, n, k, bias)
         check(lib().rt_gemm_bias_act(self._h, _dp(a), _dp(b), _dp(bias), _dp(c), m, n, k, epilogue, _dtype_code(a),
                                      _stream()))
         return c
@@ -321,6 +383,7 @@ class Gemm:
         """c = a @ bt.T (+ bias, + GELU as `epilogue` says) with the weights kept as bt[N, K]."""
         m, k = a.shape
         n = bt.shape[0]
+        self._operands(a, bt, c, m, n, k, bias)
         check(lib().rt_gemm_bt(self._h, _dp(a), _dp(bt), None if bias is None else _dp(bias), _dp(c), m, n, k, epilogue,
                                _dtype_code(a), _stream()))
         return c

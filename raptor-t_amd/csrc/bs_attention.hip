@@ -897,8 +897,11 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
     // one per wave.  Two passes over the workgroup's slice: the pipelined loop first, then, for what
     // it handed back (s_redo: one flag per plan entry of the slice, at most REDO_ENTRIES), the
     // moving-maximum loop.
-    const int begin = a.from_pos[blockIdx.x], end = a.from_pos[blockIdx.x + 1];
+    // A plan the host has not checked (rt_meta_check_partition) must not make this kernel read outside
+    // from_idx: the slice is clamped to its n_units entries, ids outside [0, n_units) are skipped.
     const int n_units = a.nb_total * a.heads;
+    const int begin = min(max(a.from_pos[blockIdx.x], 0), n_units);
+    const int end = min(max(a.from_pos[blockIdx.x + 1], begin), n_units);
     auto walk = [&](auto fast) {
       constexpr bool FAST = decltype(fast)::value;
       int p = begin;

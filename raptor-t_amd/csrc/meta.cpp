@@ -388,4 +388,25 @@ int rt_meta_partition_lpt(const int* sb, int batch, int heads, int n_wg, int* ou
   return RT_OK;
 }
 
+int rt_meta_check_partition(const int* from_pos, const int* from_idx, int n_wg, int total_blocks, int heads) {
+  RT_REQUIRE(from_pos && from_idx, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(n_wg >= 1 && total_blocks >= 1 && heads >= 1, RT_EINVAL, "bad n_wg=%d / total_blocks=%d / heads=%d", n_wg,
+             total_blocks, heads);
+  const int64_t units = int64_t(total_blocks) * heads;
+  RT_REQUIRE(units < (int64_t(1) << 31), RT_EINVAL, "too many units: %d blocks x %d heads", total_blocks, heads);
+  RT_REQUIRE(from_pos[0] == 0 && from_pos[n_wg] == units, RT_EINVAL,
+             "partition: from_pos must run from 0 to %lld, got %d .. %d", (long long)units, from_pos[0], from_pos[n_wg]);
+  for (int c = 0; c < n_wg; ++c)
+    RT_REQUIRE(from_pos[c] <= from_pos[c + 1], RT_EINVAL, "partition: from_pos decreases at workgroup %d", c);
+  std::vector<uint8_t> seen(size_t(units), 0);
+  for (int64_t i = 0; i < units; ++i) {
+    const int u = from_idx[i];
+    RT_REQUIRE(u >= 0 && u < units, RT_EINVAL, "partition: unit id %d at position %lld is outside [0, %lld)", u,
+               (long long)i, (long long)units);
+    RT_REQUIRE(!seen[u], RT_EINVAL, "partition: unit id %d is listed twice", u);
+    seen[u] = 1;
+  }
+  return RT_OK;
+}
+
 }  // extern "C"

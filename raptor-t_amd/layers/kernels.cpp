@@ -39,8 +39,50 @@ rt_gemm_ctx* shared_gemm_handle() {
 }
 
 static void require_cuda_contiguous(const torch::Tensor& t, const char* name) {
-  if (!t.is_cuda() || !t.is_contiguous())
+  if (!t.defined() || !t.is_cuda() || !t.is_contiguous())
     throw std::invalid_argument(std::string(name) + " must be a contiguous GPU tensor");
+}
+
+// Every pointer below goes to a kernel as it is: a host tensor, another dtype or fewer elements than the
+// launch reads would be a GPU memory fault, not an error code.  Checked before anything is launched.
+static void require_data(const torch::Tensor& t, const char* name, torch::ScalarType dtype, int64_t min_numel) {
+  require_cuda_contiguous(t, name);
+  if (t.scalar_type() != dtype)
+    throw std::invalid_argument(std::string(name) + " has dtype " + c10::toString(t.scalar_type()) + ", expected " +
+                                c10::toString(dtype));
+  if (t.numel() < min_numel)
+    throw std::invalid_argument(std::string(name) + " holds " + std::to_string(t.numel()) + " elements, the launch needs " +
+                                std::to_string(min_numel));
+}
+
+static void require_index(const torch::Tensor& t, const char* name, int64_t numel) {
+  require_cuda_contiguous(t, name);
+  if (t.scalar_type() != torch::kInt32) throw std::invalid_argument(std::string(name) + " must be an int32 tensor");
+  if (t.numel() != numel)
+    throw std::invalid_argument(std::string(name) + " holds " + std::to_string(t.numel()) + " entries, expected " +
+                                std::to_string(numel));
+}
+
+// The host's work plan, checked once per tensor pair (same storage, same version, same size as the pair
+// checked last: nothing to do).  Costs one device-to-host copy the first time a plan is seen.
+static void require_valid_partition(const torch::Tensor& from_idx, const torch::Tensor& from_pos, int n_wg, int block_num,
+                                    int head_num) {
+  struct Key { const void* idx; const void* pos; int64_t n_idx, n_pos; uint32_t v_idx, v_pos; };
+  static std::mutex m;
+  static Key last = {nullptr, nullptr, 0, 0, 0, 0};
+  const Key now = {from_idx.data_ptr(), from_pos.data_ptr(), from_idx.numel(), from_pos.numel(),
+                   uint32_t(from_idx._version()), uint32_t(from_pos._version())};
+  {
+    std::lock_guard<std::mutex> lk(m);
+    if (now.idx == last.idx && now.pos == last.pos && now.n_idx == last.n_idx && now.n_pos == last.n_pos &&
+        now.v_idx == last.v_idx && now.v_pos == last.v_pos)
+      return;
+  }
+  const torch::Tensor idx_h = from_idx.cpu(), pos_h = from_pos.cpu();
+  check(rt_meta_check_partition(pos_h.data_ptr<int>(), idx_h.data_ptr<int>(), n_wg, block_num, head_num),
+        "balanced attention: bad work plan");
+  std::lock_guard<std::mutex> lk(m);
+  last = now;
 }
 
 namespace {
@@ -125,8 +167,9 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
   require_cuda_contiguous(out, "out");
   if (A.dim() != 2 || B.dim() != 2) throw std::invalid_argument(name + ": operands must be matrices");
   const int64_t n = b_trans ? B.size(0) : B.size(1);
-  if (A.size(1) != (b_trans ? B.size(1) : B.size(0)) || out.numel() != A.size(0) * n)
-    throw std::invalid_argument(name + ": shape mismatch");
+  if (A.size(1) != (b_trans ? B.size(1) : B.size(0)) || out.numel() != A.size(0) * n ||
+      B.scalar_type() != A.scalar_type() || out.scalar_type() != A.scalar_type())
+    throw std::invalid_argument(name + ": shape or dtype mismatch");
   static std::map<std::string, float> no_info;
   ScopedGpuTimer timer(no_info, "MatMul");
   if (b_trans)
@@ -159,7 +202,7 @@ void MatMulBiasGelu(const torch::Tensor& A, const torch::Tensor& B, const torch:
   if (A.dim() != 2 || B.dim() != 2) throw std::invalid_argument(name + ": operands must be matrices");
   const int64_t n = b_trans ? B.size(0) : B.size(1);
   if (A.size(1) != (b_trans ? B.size(1) : B.size(0)) || out.numel() != A.size(0) * n || bias.numel() != n ||
-      bias.scalar_type() != A.scalar_type())
+      bias.scalar_type() != A.scalar_type() || B.scalar_type() != A.scalar_type() || out.scalar_type() != A.scalar_type())
     throw std::invalid_argument(name + ": shape or dtype mismatch");
   ScopedGpuTimer timer(info, "MatMul_bias_gelu");
   if (b_trans)
@@ -202,8 +245,22 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
                                    torch::Tensor& k, torch::Tensor& v, const torch::Tensor& seq_len_info_tensor,
                                    int batch_size, int head_num, int block_num, int head_size,
                                    std::map<std::string, float>& info, bool kernel_fusion) {
-  ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel");
   if (head_size != RT_HEAD_DIM) throw std::invalid_argument("head size must be 64");
+  if (batch_size < 1 || head_num < 1 || block_num < batch_size)
+    throw std::invalid_argument("add_bias_and_transpose_kernel: bad batch_size / head_num / block_num");
+  {
+    require_cuda_contiguous(input_data, "qkv");
+    const torch::ScalarType dt = input_data.scalar_type();
+    const int64_t per_tensor = int64_t(block_num) * 64 * head_num * head_size;
+    if (input_data.numel() != 3 * per_tensor)
+      throw std::invalid_argument("add_bias_and_transpose_kernel: qkv must be [block_num * 64, 3 * heads * 64]");
+    require_data(bias, "qkv bias", dt, 3 * int64_t(head_num) * head_size);
+    if (!(kernel_fusion && attention_q_from_rows())) require_data(q, "q", dt, per_tensor);
+    require_data(k, "k", dt, per_tensor);
+    require_data(v, "v", dt, per_tensor);
+    require_index(seq_len_info_tensor, "seq_len_info_tensor", int64_t(batch_size) + 1);
+  }
+  ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel");
   // the attention kernel evaluates the softmax in base 2: fold log2(e) into the Q scale
   const float scale = kQScale;
   if (kernel_fusion) {
@@ -246,6 +303,21 @@ void add_bias_and_layernorm_kernel(torch::Tensor& out, const torch::Tensor& inpu
                                    int seq_len, int normalized_len, float eps, const torch::Tensor& layernorm_weight,
                                    const torch::Tensor& layernorm_bias, std::map<std::string, float>& info,
                                    bool kernel_fusion) {
+  if (seq_len < 0 || normalized_len < 1) throw std::invalid_argument("add_bias_and_layernorm_kernel: bad seq_len / width");
+  {
+    require_cuda_contiguous(out, "out");
+    const torch::ScalarType dt = out.scalar_type();
+    const int64_t n = int64_t(seq_len) * normalized_len;
+    if (out.numel() != n)
+      throw std::invalid_argument("add_bias_and_layernorm_kernel: out holds " + std::to_string(out.numel()) +
+                                  " elements, seq_len x width is " + std::to_string(n));
+    require_data(input_data, "residual", dt, n);
+    if (input_data.numel() != n)
+      throw std::invalid_argument("add_bias_and_layernorm_kernel: the residual has other rows than out");
+    require_data(bias, "bias", dt, normalized_len);
+    require_data(layernorm_weight, "layernorm weight", dt, normalized_len);
+    require_data(layernorm_bias, "layernorm bias", dt, normalized_len);
+  }
   ScopedGpuTimer timer(info, "add_bias_and_layernorm_kernel");
   if (kernel_fusion) {
     check(rt_bias_residual_layernorm(out.data_ptr(), input_data.data_ptr(), bias.data_ptr(),
@@ -260,6 +332,12 @@ void add_bias_and_layernorm_kernel(torch::Tensor& out, const torch::Tensor& inpu
 
 void add_bias_act_kernel(const torch::Tensor& bias, torch::Tensor& out, int total_seq_len, int dim_size,
                          std::map<std::string, float>& info, bool kernel_fusion) {
+  if (total_seq_len < 0 || dim_size < 1) throw std::invalid_argument("add_bias_act_kernel: bad total_seq_len / dim_size");
+  require_cuda_contiguous(out, "out");
+  if (out.numel() != int64_t(total_seq_len) * dim_size)
+    throw std::invalid_argument("add_bias_act_kernel: out holds " + std::to_string(out.numel()) +
+                                " elements, total_seq_len x dim_size is " + std::to_string(int64_t(total_seq_len) * dim_size));
+  require_data(bias, "bias", out.scalar_type(), dim_size);
   ScopedGpuTimer timer(info, "add_bias_act_kernel");
   if (kernel_fusion) {
     check(rt_bias_gelu(out.data_ptr(), bias.data_ptr(), total_seq_len, dim_size, dtype_code(out), current_stream()),
@@ -278,6 +356,17 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
                       const int* to_select_index_position, int plan_heads, int block_limit, int block_num,
                       int head_num, std::map<std::string, float>& info, bool balanced, const torch::Tensor& seq_tokens,
                       const torch::Tensor& qkv_rows, const torch::Tensor& qkv_bias) {
+  if (batch_size < 1 || head_num < 1 || block_num < batch_size)
+    throw std::invalid_argument("sparse_attention: bad batch_size / head_num / block_num");
+  if (!to_select_index || !to_select_index_position) throw std::invalid_argument("sparse_attention: no block index");
+  const int64_t per_tensor = int64_t(block_num) * 64 * head_num * RT_HEAD_DIM;
+  require_cuda_contiguous(out, "attention out");
+  if (out.numel() != per_tensor)
+    throw std::invalid_argument("sparse_attention: out must hold block_num * 64 rows of heads * 64");
+  if (!qkv_rows.defined()) require_data(q, "q", out.scalar_type(), per_tensor);
+  require_data(k, "k", out.scalar_type(), per_tensor);
+  require_data(v, "v", out.scalar_type(), per_tensor);
+  require_index(seq_len_info_tensor, "seq_len_info_tensor", int64_t(batch_size) + 1);
   ScopedGpuTimer timer(info, "attention");
   const int* tokens = nullptr;
   if (seq_tokens.defined() && seq_tokens.numel() > 0) {
@@ -295,6 +384,10 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
     if (from_select_index.numel() != int64_t(block_num) * head_num)
       throw std::invalid_argument("balanced attention: the plan does not cover every (head, block) unit");
     if (attention_host_plan()) {
+      if (block_limit < 1) throw std::invalid_argument("balanced attention: block_limit must be positive");
+      require_index(from_select_index, "from_select_index", int64_t(block_num) * head_num);
+      require_index(from_select_index_position, "from_select_index_position", int64_t(block_limit) + 1);
+      require_valid_partition(from_select_index, from_select_index_position, block_limit, block_num, head_num);
       from_idx = from_select_index.data_ptr<int>();
       from_pos = from_select_index_position.data_ptr<int>();
       n_wg = block_limit;

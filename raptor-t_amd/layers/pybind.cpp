@@ -40,6 +40,55 @@ PYBIND11_MODULE(raptor_t, m) {
   m.def("attention_q_from_rows", &layers::kernels::attention_q_from_rows);
   m.def("timing_collect", &layers::kernels::timing_collect,
         "Synchronise and return {launcher: (total microseconds, launches)} since timing_begin().");
+  // The tensor-level launchers the layer objects call, under the reference's names (layers/kernels/kernel.h):
+  // for callers that drive single kernels, and so that their argument checks can be exercised without a GPU.
+  {
+    namespace k = layers::kernels;
+    using Info = std::map<std::string, float>;
+    py::module_ km = m.def_submodule("kernels", "tensor-level launchers (layers/kernels/kernel.h of the reference)");
+    km.def("add_bias_and_transpose_kernel",
+           [](const torch::Tensor& bias, torch::Tensor& qkv, torch::Tensor& q, torch::Tensor& kk, torch::Tensor& v,
+              const torch::Tensor& seq_len_info, int batch, int heads, int block_num, int head_size, bool fusion) {
+             Info info;
+             k::add_bias_and_transpose_kernel(bias, qkv, q, kk, v, seq_len_info, batch, heads, block_num, head_size, info, fusion);
+           },
+           py::arg("bias"), py::arg("qkv"), py::arg("q"), py::arg("k"), py::arg("v"), py::arg("seq_len_info_tensor"),
+           py::arg("batch_size"), py::arg("head_num"), py::arg("block_num"), py::arg("head_size") = 64,
+           py::arg("kernel_fusion") = true);
+    km.def("add_bias_and_layernorm_kernel",
+           [](torch::Tensor& out, const torch::Tensor& residual, const torch::Tensor& bias, int seq_len, int width, float eps,
+              const torch::Tensor& gamma, const torch::Tensor& beta, bool fusion) {
+             Info info;
+             k::add_bias_and_layernorm_kernel(out, residual, bias, seq_len, width, eps, gamma, beta, info, fusion);
+           },
+           py::arg("out"), py::arg("input_data"), py::arg("bias"), py::arg("seq_len"), py::arg("normalized_len"),
+           py::arg("eps"), py::arg("layernorm_weight"), py::arg("layernorm_bias"), py::arg("kernel_fusion") = true);
+    km.def("add_bias_act_kernel",
+           [](const torch::Tensor& bias, torch::Tensor& out, int rows, int width, bool fusion) {
+             Info info;
+             k::add_bias_act_kernel(bias, out, rows, width, info, fusion);
+           },
+           py::arg("bias"), py::arg("out"), py::arg("total_seq_len"), py::arg("dim_size"), py::arg("kernel_fusion") = true);
+    km.def("sparse_attention",
+           [](const torch::Tensor& q, const torch::Tensor& kk, const torch::Tensor& v, torch::Tensor& out, int batch,
+              const torch::Tensor& seq_len_info, const torch::Tensor& from_idx, const torch::Tensor& from_pos,
+              const torch::Tensor& to_idx, const torch::Tensor& to_pos, int plan_heads, int block_limit, int block_num,
+              int heads, bool balanced) {
+             for (const torch::Tensor* t : {&to_idx, &to_pos})
+               if (!t->defined() || !t->is_cuda() || !t->is_contiguous() || t->scalar_type() != torch::kInt32)
+                 throw std::invalid_argument("sparse_attention: the block index must be contiguous int32 GPU tensors");
+             if ((plan_heads != 1 && plan_heads != heads) || to_pos.numel() != int64_t(plan_heads) * block_num + 1)
+               throw std::invalid_argument("sparse_attention: to_select_index_position must hold plan_heads * block_num + 1 entries");
+             Info info;
+             k::sparse_attention(q, kk, v, out, batch, seq_len_info, from_idx, from_pos, to_idx.data_ptr<int>(),
+                                 to_pos.data_ptr<int>(), plan_heads, block_limit, block_num, heads, info, balanced);
+           },
+           py::arg("q"), py::arg("k"), py::arg("v"), py::arg("out"), py::arg("batch_size"), py::arg("seq_len_info_tensor"),
+           py::arg("from_select_index"), py::arg("from_select_index_position"), py::arg("to_select_index"),
+           py::arg("to_select_index_position"), py::arg("plan_heads"), py::arg("block_limit"), py::arg("block_num"),
+           py::arg("head_num"), py::arg("balanced") = false);
+  }
+
   py::class_<layers::BertAttention>(m, "BertAttention")
       .def(py::init([](torch::Tensor& qkv_weight, torch::Tensor& qkv_bias, torch::Tensor& dense_weight,
                        torch::Tensor& dense_bias, torch::Tensor& layer_norm_weight, torch::Tensor& layer_norm_bias,

@@ -42,3 +42,25 @@ def test_hbm_roofline_arithmetic():
     assert abs(r["achieved"] - 4000.0) < 1e-9 and abs(r["frac"] - 0.5) < 1e-12
     assert r["traffic"] == 9e6 and r["bytes_per_launch"] == 8_000_000
     json.dumps(r)
+
+
+def test_cpu_baseline_helpers():
+    """The thread count of the CPU baselines never exceeds what the job may use, and the bounded timer stops at its
+    budget but not before three runs."""
+    b = _bench()
+    n = b.host_cores()
+    assert 1 <= n <= (os.cpu_count() or 1)
+    old = os.environ.get("OMP_NUM_THREADS")
+    os.environ["OMP_NUM_THREADS"] = "1"
+    try:
+        assert b.host_cores() == 1
+    finally:
+        if old is None:
+            del os.environ["OMP_NUM_THREADS"]
+        else:
+            os.environ["OMP_NUM_THREADS"] = old
+    calls = []
+    med, runs = b.timed_median(lambda: calls.append(1), warmup=2, reps=50, budget_s=0.0)
+    assert runs == 3 and len(calls) == 5 and med >= 0.0
+    med, runs = b.timed_median(lambda: None, warmup=0, reps=4, budget_s=60.0)
+    assert runs == 4

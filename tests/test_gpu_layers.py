@@ -11,6 +11,7 @@ import torch
 import __graft_entry__ as graft
 from oracle import layer as ol
 from oracle import metadata as md
+from tests import layer_harness as lh
 
 pytestmark = pytest.mark.gpu
 
@@ -37,13 +38,18 @@ def say(*a):
     print(*a, flush=True)
 
 
-def _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype):
+def _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype, max_pos=4096):
+    """bf16: the oracle rounds every tensor that passes between two kernels to bf16, as the layer objects (and the
+    reference, in its fp16) store them; with 8 mantissa bits these roundings, not the kernels' arithmetic, decide
+    the distance to an all-fp32 layer (0.04 after two layers), and a bound that lets them through would hide a real
+    error at small |y|.  fp16 is compared with the all-fp32 layer."""
     sb = md.seq_prefix_blocks(seq_lens)
     h = x32.to(dtype).float()
+    store = dtype if dtype == torch.bfloat16 else None
     for li, w in enumerate(layers_w32):
         wr = {k: v.to(dtype).float() for k, v in w.items()}
-        idx, pos = md.hf_to_index(seq_lens, li, heads)
-        h = ol.encoder_layer(h, wr, heads, sb, idx, pos, heads, eps)
+        idx, pos = md.hf_to_index(seq_lens, li, heads, max_pos=max_pos)
+        h = ol.encoder_layer(h, wr, heads, sb, idx, pos, heads, eps, store_dtype=store)
     return h
 
 
@@ -60,7 +66,6 @@ def test_encoder_through_layer_api_matches_oracle(mb, ut, async_, balanced, dtyp
     layers_w = [{k: v.to(dtype).cuda() for k, v in w.items()} for w in layers_w32]
     enc = mb.BertEncoder.from_weights(layers_w, heads, async_=async_, eps=eps)
     meta = mb.cxx.MetaData()
-    worst = 0.0
     mb.cxx.set_attention_host_plan(balanced)               # balanced: walk the host's LPT partition, as the reference does
     for seq_lens in ([832, 1024, 256], [1280, 768]):       # two batches through the same objects
         t = sum(seq_lens)
@@ -77,12 +82,82 @@ def test_encoder_through_layer_api_matches_oracle(mb, ut, async_, balanced, dtyp
         assert out.data_ptr() == hidden_states.data_ptr()       # FFN writes back into the layer input buffer
         assert info["attention"] > 0.0 and info["pre_process"] >= 0.0
         want = _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype)
-        err = (out.float().cpu() - want).abs().max().item()
-        say("  err", err, "info", info)
-        worst = max(worst, err)
+        say("  err", (out.float().cpu() - want).abs().max().item(), "info", info)
+        lh.check_stack_output(out, want, dtype)
     mb.cxx.set_attention_host_plan(False)
     meta.terminate_thread()
-    assert worst <= (2e-2 if dtype == torch.float16 else 8e-2)   # bf16: one ulp at |y| ~ 4 is 3e-2
+
+
+def test_large_configuration_geometry_through_layer_api(pkg, mb, ut):
+    """The large configuration's geometry at batch 2 (hidden 1024, 16 heads, FFN 4096, bf16, sequences of 8192 and
+    4160 tokens: global rows of 128 and 65 key blocks) through the layer objects with the block-index pipeline
+    on and the plans drawn for 16384 positions, against the oracle."""
+    say("large configuration via layer api")
+    hidden, heads, ffn, dtype, eps, block_limit = 1024, 16, 4096, torch.bfloat16, 1e-5, 128
+    seq_lens = [8192, 4160]
+    g = torch.Generator().manual_seed(3)
+    layers_w32 = [ol.random_layer_weights(hidden, ffn, g) for _ in range(2)]
+    layers_w = [{k: v.to(dtype).cuda() for k, v in w.items()} for w in layers_w32]
+    mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, 16384)
+    try:
+        enc = mb.BertEncoder.from_weights(layers_w, heads, async_=True, eps=eps)
+        meta = mb.cxx.MetaData()
+        t = sum(seq_lens)
+        x32 = torch.randn(t, hidden, generator=g)
+        hidden_states = x32.to(dtype).cuda()
+        spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, block_limit, heads)
+        meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+        new = lambda w: torch.empty(t, w, dtype=dtype, device="cuda")
+        out, _ = enc(hidden_states, t, block_limit, spi, spi_t, ppi_t, pp_t, new(hidden), new(ffn), new(hidden))
+        torch.cuda.synchronize()
+        meta.terminate_thread()
+    finally:
+        mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, 4096)
+    assert torch.isfinite(out.float()).all()
+    want = _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype, max_pos=16384)
+    say("  err", (out.float().cpu() - want).abs().max().item())
+    lh.check_stack_output(out, want, dtype)
+
+
+def test_launchers_refuse_mismatched_gpu_tensors(pkg, mb):
+    """On the GPU the same checks see real device tensors: an int64 index tensor, a residual with other rows than the
+    output, a K shorter than the launch reads and a work plan with an id out of range are refused before any launch."""
+    say("launcher argument checks")
+    k, capi = mb.cxx.kernels, pkg.capi
+    heads, nb = 2, 14
+    t = nb * 64
+    h = lambda *shape: torch.zeros(*shape, dtype=torch.float16, device="cuda")
+    sb = torch.tensor([0, nb], dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="int32"):
+        k.add_bias_and_transpose_kernel(h(3 * heads * 64), h(t, 3 * heads * 64), h(t * heads * 64), h(t * heads * 64),
+                                        h(t * heads * 64), sb.long(), 1, heads, nb)
+    with pytest.raises(ValueError, match="residual"):
+        k.add_bias_and_layernorm_kernel(h(t, 128), h(t - 64, 128), h(128), t, 128, 1e-5, h(128), h(128))
+    with pytest.raises(ValueError, match="dtype"):
+        k.add_bias_act_kernel(h(128).float(), h(t, 128), t, 128)
+    idx, pos = capi.build_to_index(sb.cpu().numpy(), heads)
+    idx_d, pos_d = torch.from_numpy(idx).cuda(), torch.from_numpy(pos).cuda()
+    fp, fi = capi.partition_lpt(sb.cpu().numpy(), heads, 4)
+    fp_d, fi_d = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
+    q, kk, v, out = h(t * heads * 64), h(t * heads * 64), h(t * heads * 64), h(t, heads * 64)
+    with pytest.raises(ValueError, match="k holds"):
+        k.sparse_attention(q, kk[:-64], v, out, 1, sb, fi_d, fp_d, idx_d, pos_d, heads, 4, nb, heads, False)
+    mb.cxx.set_attention_host_plan(True)
+    try:
+        k.sparse_attention(q, kk, v, out, 1, sb, fi_d, fp_d, idx_d, pos_d, heads, 4, nb, heads, True)     # a good plan runs
+        bad = fi_d.clone()
+        bad[3] = nb * heads
+        with pytest.raises(RuntimeError, match="outside"):
+            k.sparse_attention(q, kk, v, out, 1, sb, bad, fp_d, idx_d, pos_d, heads, 4, nb, heads, True)
+        fi_d[0] = -7                                         # the same tensor changed in place is checked again
+        with pytest.raises(RuntimeError, match="outside"):
+            k.sparse_attention(q, kk, v, out, 1, sb, fi_d, fp_d, idx_d, pos_d, heads, 4, nb, heads, True)
+    finally:
+        mb.cxx.set_attention_host_plan(False)
+    torch.cuda.synchronize()
+    with pytest.raises(ValueError, match="dtype"):
+        capi.bs_attention_fwd(q, kk, v, out, sb.long(), heads, idx_d, pos_d, heads)
+    assert torch.isfinite(out).all()
 
 
 def test_fused_and_unfused_paths_agree(mb, ut):
