@@ -1,6 +1,6 @@
 """Benchmark of the block-sparse encoder hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|ref_e2e|stream]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2|c4|c5|ref_e2e|stream]
 
 Default workload `c3` is the headline configuration (benchmark config 3): the 12-layer BigBird-base fp16 encoder
 on a padding-free batch of 16 sequences with lengths uniform in [512, 4096] (multiples of
@@ -27,7 +27,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 import __graft_entry__ as graft  # noqa: E402
 
-MFMA_PEAK = {"f16": 2.5e15, "bf16": 2.5e15}       # MI355X dense matrix peak, FLOP/s
+MFMA_PEAK = {"f16": 2.5e15, "bf16": 2.5e15, "f32": 157.3e12}       # MI355X dense matrix peak, FLOP/s
 HBM_PEAK = 8.0e12                                   # B/s
 PAIR_FLOP = 4 * 64 * 64 * 64                        # QK^T + PV of one (from-block, to-block) pair, d = 64
 METRIC = "seqs/sec + ms/layer, BigBird-base fp16 var-len<=4096; attn MFMA %, LN HBM GB/s"
@@ -194,7 +194,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
     pkg = graft.load_package()
     mb = importlib.import_module("raptor_t_amd.modeling_bert")
     ut = importlib.import_module("raptor_t_amd.util")
-    dt = {"f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    dt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
     g = torch.Generator().manual_seed(0)
     layers_w = [mb.random_layer_weights(hidden, ffn, g, dtype=dt) for _ in range(layers)]
     mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, max_pos)
@@ -252,7 +252,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
     att_us = per["attention"]
     att_flops = pairs * PAIR_FLOP
     ach = att_flops / (att_us * 1e-6)
-    sz = 2
+    sz = 4 if dtype == "f32" else 2
     traffic = MEASURED_TRAFFIC_C3 if name.startswith("c3") else {}
     out = {
         "metric": METRIC, "value": len(seq_lens) / (elapsed / args.steps), "unit": "seqs/s", "n_gpus": 1,
@@ -446,7 +446,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c2", "c4", "c5", "ref_e2e", "stream"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c1", "c2", "c4", "c5", "ref_e2e", "stream"])
     ap.add_argument("--block-limit", type=int, default=1024, help="persistent workgroups of the balanced attention launch")
     ap.add_argument("--lpt-plan", action="store_true",
                     help="drive attention with the caller's LPT plan (the reference's balanced mode) instead of the kernel's own schedule")
@@ -472,6 +472,9 @@ def main():
     if args.workload == "c3":
         res = run_encoder(args, "c3: 12-layer BigBird-base, batch 16, len U[512,4096]", 768, 12, 3072, 12, "f16",
                           ut.uniform_lengths(16, 512, 4096, seed=0))
+    elif args.workload == "c1":
+        res = run_encoder(args, "c1: one BigBird-base layer, batch 1 x 1024 tokens, fp32 (the accuracy mode)", 768, 12,
+                          3072, 1, "f32", [1024])
     elif args.workload == "c5":
         res = run_encoder(args, "c5: 24-layer BigBird-large shape, batch 4, len U[2048,16384], bf16", 1024, 16, 4096,
                           24, "bf16", ut.uniform_lengths(4, 2048, 16384, seed=0), max_pos=16384)

@@ -136,8 +136,16 @@ int rt_unpack_head_tiles(const void* packed, void* dst, const int* seq_blocks_de
  * as 2^(q.k) / sum 2^(q.k): the scale log2(e)/sqrt(d) is already folded into q.  to_idx/to_pos: device CSR from rt_meta_build_to_index
  * (plan_heads = 1 or heads).  If from_idx/from_pos are non-NULL the launch is
  * `n_wg` persistent workgroups each walking its slice of the LPT plan (balanced);
- * otherwise the kernel enumerates the units itself (global rows first inside each
- * (sequence, head) group, XCD-contiguous order). */
+ * otherwise the kernel hands the units out itself: two persistent workgroups per CU draw
+ * tickets from per-XCD counters, the two rows of each sparse (sequence, head) that list every
+ * block first (four waves share such a row), then one unit per wave.
+ * dtype RT_F16 / RT_BF16: fp32 accumulation, probabilities rounded to the tensor type for the
+ * second product.  RT_F32 (the reference's fp32-output dispatch, sparse_attention.cu:1582-1599):
+ * every tensor fp32, fp32 matrix instructions; an accuracy mode, about ten times slower.
+ * Limits of one launch (RT_EINVAL beyond them): batch <= 1024 sequences, total_blocks <= 4096
+ * (262144 tokens), total_blocks * heads * 24576 < 2^31 (byte offsets are 32-bit).  The first launch
+ * on a device without from_idx/from_pos allocates 256 KiB of counters that the library keeps
+ * (rt_bs_attention_fwd_no_alloc does not). */
 int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out,
                         const int* seq_blocks_dev, int batch, int total_blocks, int heads,
                         const int* to_idx, const int* to_pos, int plan_heads,
@@ -162,7 +170,8 @@ int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, voi
  * the same fp32 arithmetic and rounding as the split kernel, so both routes give the same bits).
  * k and vt still come from rt_qkv_bias_split (called with q = NULL).  Same stage of the
  * reference as rt_bs_attention_fwd; the reference always materialises Q
- * (layers/kernels/add_bias_and_transpose.cu:212-233).  seq_tokens_dev may be NULL. */
+ * (layers/kernels/add_bias_and_transpose.cu:212-233).  seq_tokens_dev may be NULL.
+ * At most 64 heads. */
 int rt_bs_attention_fwd_qrows(const void* qkv, const void* qkv_bias, float q_scale, const void* k,
                               const void* vt, void* out, const int* seq_blocks_dev,
                               const int* seq_tokens_dev, int batch, int total_blocks, int heads,

@@ -1183,8 +1183,12 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
   RT_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(q_rows) | reinterpret_cast<uintptr_t>(q_bias) |
                reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(vt) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0,
              RT_EINVAL, "q (or qkv and its bias), k, vt, out must be 16-byte aligned");
-  if (dtype == RT_F32) return rt::fail(RT_ENOSYS, "block-sparse attention runs in fp16 or bf16 (fp32 accumulation)");
-  RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16, RT_EINVAL, "unknown dtype %d", dtype);
+  RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);
+  if (dtype == RT_F32) {
+    RT_REQUIRE(!from_idx || n_wg >= 1, RT_EINVAL, "balanced launch needs n_wg >= 1, got %d", n_wg);
+    return rt::launch_attention_f32(q, q_rows, q_bias, q_scale, k, vt, out, seq_blocks_dev, seq_tokens_dev, batch,
+                                    total_blocks, heads, to_idx, to_pos, plan_heads, from_idx, from_pos, n_wg, stream);
+  }
   unsigned grid;
   int* queues = nullptr;
   int* queues_clear = nullptr;

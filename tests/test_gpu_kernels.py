@@ -118,7 +118,7 @@ def test_qkv_bias_split_layout_bit_exact(capi, dtype):
     assert torch.equal(k2, k) and torch.equal(vt2, vt)
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("lens,heads,n_wg", [
     ([768], 2, 0), ([1024, 64, 832, 512], 3, 0), ([1024, 64, 832, 512], 3, 7), ([2048, 768], 12, 160),
     ([64], 1, 0), ([128, 192], 2, 3),
@@ -146,6 +146,59 @@ def test_attention_rows_longer_than_64_blocks(capi, n_wg):
     out, ref = lh.run_attention(capi, q, k, v, lens, heads, seed=4, n_wg=n_wg, max_pos=16384)
     assert not torch.isnan(out).any()
     assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("n_wg,padded,from_rows", [(0, False, False), (5, True, False), (0, True, True), (9, False, True)])
+def test_attention_fp32_mode(capi, n_wg, padded, from_rows):
+    """The fp32 instantiation (the layer's accuracy mode; config 1 of the benchmark runs in it) to 1e-4: a sparse
+    sequence, a short one, a global row of more than 64 key blocks, padded tails, queries taken from the projection's
+    rows, with and without a work plan."""
+    say("attention fp32", n_wg, padded, from_rows)
+    heads, seq_lens = 3, [64 * 13, 64 * 3, 64 * 66, 64]
+    t, dm = sum(seq_lens), heads * 64
+    g = torch.Generator().manual_seed(15)
+    qkv = torch.randn(t, 3 * dm, generator=g).cuda()
+    bias = (torch.randn(3 * dm, generator=g) * 0.5).cuda()
+    sb, idx, pos, ph, sb_d, idx_d, pos_d = lh.device_plan(capi, seq_lens, heads, 2, None, max_pos=16384)
+    seq_tokens = [n - 23 for n in seq_lens] if padded else None
+    tok_d = None if seq_tokens is None else torch.tensor(seq_tokens, dtype=torch.int32).cuda()
+    from_idx = from_pos = None
+    if n_wg:
+        fp, fi = capi.partition_lpt(sb, heads, n_wg)
+        from_pos, from_idx = torch.from_numpy(fp).cuda(), torch.from_numpy(fi).cuda()
+    new = lambda: torch.full((t * dm,), float("nan"), device="cuda")
+    q, k, vt, out = new(), new(), new(), new().view(t, dm)
+    if from_rows:
+        capi.qkv_bias_split(qkv, bias, None, k, vt, sb_d, heads, capi.Q_SCALE)
+        capi.bs_attention_fwd_qrows(qkv, bias, capi.Q_SCALE, k, vt, out, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos,
+                                    tok_d)
+    else:
+        capi.qkv_bias_split(qkv, bias, q, k, vt, sb_d, heads, capi.Q_SCALE)
+        capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos, tok_d)
+    torch.cuda.synchronize()
+    x = qkv.cpu() + bias.cpu()
+    qs = (x[:, :dm] * capi.Q_SCALE).view(t, heads, 64)
+    kk, vv = (x[:, i * dm:(i + 1) * dm].view(t, heads, 64) for i in (1, 2))
+    ref = oa.csr_attention(qs, kk, vv, sb.tolist(), idx, pos, ph, scale=1.0 / lh.LOG2E, seq_tokens=seq_tokens)
+    rows = torch.ones(t, dtype=torch.bool)
+    if padded:                                             # padded query rows are computed but not specified
+        start = 0
+        for n, real in zip(seq_lens, seq_tokens):
+            rows[start + real:start + n] = False
+            start += n
+    assert torch.isfinite(out).all()
+    assert (out.cpu()[rows] - ref[rows]).abs().max().item() <= 1e-4
+
+
+def test_encoder_layer_config1_fp32(capi):
+    """Benchmark config 1 on the GPU path: one BigBird-base layer, batch 1, 1024 tokens, hidden 768, 12 heads, FFN 3072,
+    every tensor fp32, against the oracle to 1e-4."""
+    say("layer config 1 fp32")
+    pkg = graft.load_package()
+    out, want = lh.run_layer_case_tensors(pkg, [1024], 768, 12, 3072, torch.float32, seed=0)
+    err = (out - want).abs().max().item()
+    say("  err", err)
+    assert err <= 1e-4
 
 
 @pytest.mark.parametrize("n_wg", [0, 128])

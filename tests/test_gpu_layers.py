@@ -57,6 +57,7 @@ def _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype, max_pos=4096):
     (True, True, torch.float16, 768, 12, 3072),
     (False, False, torch.float16, 768, 12, 3072),
     (True, True, torch.bfloat16, 1024, 16, 4096),
+    (True, False, torch.float32, 768, 12, 3072),
 ])
 def test_encoder_through_layer_api_matches_oracle(mb, ut, async_, balanced, dtype, hidden, heads, ffn):
     say("encoder api", async_, balanced, dtype, hidden)
