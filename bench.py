@@ -289,9 +289,12 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
 
 
 def time_kernel(fn, steps, warmup, settle_ms=25.0):
-    """Median duration of one launch in microseconds.  After the warm-up launches the kernel keeps running
+    """Median GPU duration of one launch in microseconds.  After the warm-up launches the kernel keeps running
     for `settle_ms`: from idle the GPU takes some tens of launches to reach its sustained clocks (the first
-    launches of a 100 us kernel measure 10-15 % slow), and a kernel inside a running job never sees that ramp."""
+    launches of a 100 us kernel measure 10-15 % slow), and a kernel inside a running job never sees that ramp.
+    The timed launches are queued behind a spin kernel that keeps the GPU busy while the host enqueues all of
+    them: a launch through Python costs the host about 10 us, more than a small kernel runs, and an idle GPU
+    waiting for its next launch would be timed as part of it."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -300,7 +303,12 @@ def time_kernel(fn, steps, warmup, settle_ms=25.0):
         for _ in range(10):
             fn()
         torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    fn()
+    host_us = (time.perf_counter() - t0) * 1e6                 # what one enqueue costs the host
+    torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda._sleep(int(2.4e3 * (3.0 * host_us + 20.0) * steps))   # cycles: three times the host's enqueue time
     for a, b in evs:
         a.record()
         fn()
@@ -347,32 +355,51 @@ def run_attention_only(args):
 
 
 def run_membound_sweep(args):
-    """Benchmark config 4: LayerNorm and GELU epilogues over tokens {8K, 32K, 64K}, fp16 and bf16."""
+    """Benchmark config 4: LayerNorm and GELU epilogues over tokens {8K, 32K, 64K}, fp16 and bf16.
+    Every kernel is timed twice: `frac` with its launches rotating over enough separate buffers that no launch finds
+    its operands where an earlier one left them (the rotation covers more than 600 MB; the memory-side cache holds
+    256 MB), and `frac_resident` with every launch on the same buffers, as a loop over one tensor runs it."""
     capi = graft.load_package().capi
     rows = []
+
+    def rotating(make, call, set_bytes):
+        sets = [make() for _ in range(max(2, -(-600_000_000 // set_bytes) + 1))]
+        state = [0]
+
+        def fn():
+            state[0] = (state[0] + 1) % len(sets)
+            call(*sets[state[0]])
+        cold = time_kernel(fn, args.steps, args.warmup)
+        warm = time_kernel(lambda: call(*sets[0]), args.steps, args.warmup)
+        for st in sets:
+            assert bool(torch.isfinite(st[0]).all()), "output is not finite"
+        return cold, warm
+
     for dt, name in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
         for t in (8192, 32768, 65536):
             g = torch.Generator(device="cuda").manual_seed(0)
             rn = lambda *s: torch.randn(*s, generator=g, device="cuda").to(dt)
-            x, r, b, ga, be = rn(t, 768), rn(t, 768), rn(768), rn(768), rn(768)
-            us = time_kernel(lambda: capi.bias_residual_layernorm(x, r, b, ga, be, 1e-5), args.steps, args.warmup)
-            rows.append(dict(hbm_roofline("bias_residual_layernorm_kernel", 3 * t * 768 * 2, us), tokens=t, dtype=name, us=us))
-            y, b2 = rn(t, 3072), rn(3072)
-            us = time_kernel(lambda: capi.bias_gelu(y, b2), args.steps, args.warmup)
-            rows.append(dict(hbm_roofline("bias_gelu_kernel", 2 * t * 3072 * 2, us), tokens=t, dtype=name, us=us))
+            b, ga, be, b2 = rn(768), rn(768), rn(768), rn(3072)
+            us, warm = rotating(lambda: (rn(t, 768), rn(t, 768)),
+                                lambda x, r: capi.bias_residual_layernorm(x, r, b, ga, be, 1e-5), 2 * t * 768 * 2)
+            rows.append(dict(hbm_roofline("bias_residual_layernorm_kernel", 3 * t * 768 * 2, us), tokens=t, dtype=name, us=us,
+                             us_resident=warm, frac_resident=3 * t * 768 * 2 / (warm * 1e-6) / HBM_PEAK))
+            us, warm = rotating(lambda: (rn(t, 3072),), lambda y: capi.bias_gelu(y, b2), t * 3072 * 2)
+            rows.append(dict(hbm_roofline("bias_gelu_kernel", 2 * t * 3072 * 2, us), tokens=t, dtype=name, us=us,
+                             us_resident=warm, frac_resident=2 * t * 3072 * 2 / (warm * 1e-6) / HBM_PEAK))
             # packed-input front end: fp32 tables (BigBird vocabulary 50358, 4096 positions), output in dt; per
             # token one fp32 word row read and one output row written (position / type rows recur and stay cached)
             gi = torch.Generator().manual_seed(0)
             word, pos, typ = (torch.randn(n, 768, generator=gi).cuda() for n in (50358, 4096, 2))
             ga32, be32 = torch.ones(768, device="cuda"), torch.zeros(768, device="cuda")
-            ids = torch.randint(0, 50358, (t,), generator=gi, dtype=torch.int32).cuda()
             pids = (torch.arange(t, dtype=torch.int32) % 4096).cuda()
             tids = torch.zeros(t, dtype=torch.int32, device="cuda")
-            e = torch.empty(t, 768, dtype=dt, device="cuda")
-            us = time_kernel(lambda: capi.embed_layernorm(ids, pids, tids, word, pos, typ, ga32, be32, e), args.steps, args.warmup)
-            rows.append(dict(hbm_roofline("embed_layernorm_kernel", t * 768 * (4 + 2), us), tokens=t, dtype=name, us=us))
-            for nm, buf in (("LayerNorm", x), ("GELU", y), ("embedding", e)):
-                assert bool(torch.isfinite(buf).all()), "%s output at %d tokens is not finite" % (nm, t)
+            us, warm = rotating(lambda: (torch.empty(t, 768, dtype=dt, device="cuda"),
+                                         torch.randint(0, 50358, (t,), generator=gi, dtype=torch.int32).cuda()),
+                                lambda e, ids: capi.embed_layernorm(ids, pids, tids, word, pos, typ, ga32, be32, e),
+                                t * 768 * (4 + 2))
+            rows.append(dict(hbm_roofline("embed_layernorm_kernel", t * 768 * (4 + 2), us), tokens=t, dtype=name, us=us,
+                             us_resident=warm, frac_resident=t * 768 * (4 + 2) / (warm * 1e-6) / HBM_PEAK))
     best_ln = max(r["frac"] for r in rows if r["kernel"].startswith("bias_residual"))
     res = {"metric": "fused add-bias+LayerNorm / bias+GELU achieved HBM GB/s", "value": best_ln * 8000.0, "unit": "GB/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
