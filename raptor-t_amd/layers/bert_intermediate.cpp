@@ -11,11 +11,11 @@ BertIntermediate::BertIntermediate(torch::Tensor dense_weight, torch::Tensor den
     throw std::invalid_argument("BertIntermediate: weight must be [D, F] and bias [F]");
   // kept as [F, D]: the GEMM is faster with both operands contiguous along the reduction
   dense_weight_ = dense_weight_.t().contiguous();
-  handle_ = kernels::shared_gemm_handle();
 }
 
 std::map<std::string, float> BertIntermediate::operator()(const torch::Tensor& input_tensor, torch::Tensor& output_tensor,
                                                           std::map<std::string, float>& info, bool kernel_fusion) const {
+  rt_gemm_ctx* const handle_ = kernels::shared_gemm_handle();       // the current micro-batch lane's workspace
   if (kernel_fusion && kernels::gemm_epilogue_fusion()) {
     kernels::MatMulBiasGelu(input_tensor, dense_weight_, dense_bias_, output_tensor, handle_, info, "BertIntermediate",
                             true);

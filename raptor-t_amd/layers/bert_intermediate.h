@@ -19,7 +19,6 @@ class BertIntermediate {
 
  private:
   torch::Tensor dense_weight_, dense_bias_;
-  rt_gemm_ctx* handle_;
 };
 
 }  // namespace layers

@@ -14,13 +14,13 @@ BertOutput::BertOutput(torch::Tensor dense_weight, torch::Tensor dense_bias, tor
       layer_norm_weight_.numel() != dense_weight_.size(1) || layer_norm_bias_.numel() != dense_weight_.size(1))
     throw std::invalid_argument("BertOutput: weight must be [F, D], bias / gamma / beta [D]");
   dense_weight_ = dense_weight_.t().contiguous();      // kept as [D, F], see BertIntermediate
-  handle_ = kernels::shared_gemm_handle();
 }
 
 std::map<std::string, float> BertOutput::operator()(const torch::Tensor& hidden_states, const torch::Tensor& input_tensor,
                                                     torch::Tensor& output_tensor, std::map<std::string, float>& info,
                                                     bool kernel_fusion) const {
-  kernels::MatMul(hidden_states, false, dense_weight_, true, 1.0, output_tensor, 0.0, handle_, "BertOutput");
+  kernels::MatMul(hidden_states, false, dense_weight_, true, 1.0, output_tensor, 0.0, kernels::shared_gemm_handle(),
+                  "BertOutput");
   const int seq_len = int(input_tensor.size(0));
   kernels::add_bias_and_layernorm_kernel(output_tensor, input_tensor, dense_bias_, seq_len, int(dense_weight_.size(0)),
                                          eps_, layer_norm_weight_, layer_norm_bias_, info, kernel_fusion);

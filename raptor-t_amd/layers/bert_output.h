@@ -24,7 +24,6 @@ class BertOutput {
  private:
   torch::Tensor dense_weight_, dense_bias_, layer_norm_weight_, layer_norm_bias_;
   float eps_;
-  rt_gemm_ctx* handle_;
 };
 
 }  // namespace layers

@@ -32,10 +32,11 @@ void check(int rc, const char* what) {
 
 rt_gemm_ctx* shared_gemm_handle() {
   static std::mutex m;
-  static rt_gemm_ctx* ctx = nullptr;
+  static rt_gemm_ctx* ctx[LANES] = {};
+  const int lane = current_lane();
   std::lock_guard<std::mutex> lk(m);
-  if (!ctx) check(rt_gemm_create(&ctx), "rt_gemm_create");
-  return ctx;
+  if (!ctx[lane]) check(rt_gemm_create(&ctx[lane]), "rt_gemm_create");
+  return ctx[lane];
 }
 
 static void require_cuda_contiguous(const torch::Tensor& t, const char* name) {
@@ -92,14 +93,19 @@ struct Deferred {
   struct Rec { std::string key; hipEvent_t a, b; };
   std::vector<Rec> recs;
   std::set<std::string> only;          // empty: every launcher is timed
+  int every = 1;                       // of a launcher's calls, one in `every` is bracketed
+  std::map<std::string, int64_t> calls;
 };
 Deferred& deferred() { static Deferred d; return d; }
 }  // namespace
 
-void timing_begin(const std::vector<std::string>& only) {
+void timing_begin(const std::vector<std::string>& only, int every) {
+  if (every < 1) throw std::invalid_argument("timing_begin: every must be at least 1");
   Deferred& d = deferred();
   std::lock_guard<std::mutex> lk(d.m);
   d.only = std::set<std::string>(only.begin(), only.end());
+  d.every = every;
+  d.calls.clear();
   for (auto& r : d.recs) { (void)hipEventDestroy(r.a); (void)hipEventDestroy(r.b); }
   d.recs.clear();
   d.active = true;
@@ -131,6 +137,7 @@ ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* k
     Deferred& d = deferred();
     std::lock_guard<std::mutex> lk(d.m);
     deferred_ = d.active && (d.only.empty() || d.only.count(key) != 0);
+    if (deferred_ && d.every > 1) deferred_ = (d.calls[key]++ % d.every) == 0;
   }
   if (!slot_ && !deferred_) return;
   hipEvent_t a, b;

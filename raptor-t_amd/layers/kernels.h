@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "../../include/raptor_t_hip.h"
+#include "tensor_set.h"
 
 namespace sparse_transformers {
 namespace layers {
@@ -24,8 +25,9 @@ enum class ActivationType { Gelu = 0, Tanh = 1, Relu = 2 };
 void* current_stream();
 int dtype_code(const torch::Tensor& t);
 void check(int rc, const char* what);
-// One hipBLASLt context (heuristic cache + workspace) shared by every layer of the process;
-// the reference creates a cuBLAS handle per layer object (multi_headed_attention.h:94).
+// One hipBLASLt context (heuristic cache + workspace) per micro-batch lane (tensor_set.h), shared by every
+// layer of the process; the reference creates a cuBLAS handle per layer object (multi_headed_attention.h:94).
+// Two lanes run on two streams at once and must not share a workspace.
 rt_gemm_ctx* shared_gemm_handle();
 
 // Deferred timing: between timing_begin() and timing_collect() every launcher below
@@ -33,7 +35,9 @@ rt_gemm_ctx* shared_gemm_handle();
 // synchronising; timing_collect() synchronises once and returns, per launcher name,
 // (total microseconds, number of launches).  Lets a harness time kernels inside an
 // otherwise free-running loop.
-void timing_begin(const std::vector<std::string>& only = {});
+// `every` > 1 brackets only one in `every` calls of each launcher: a pair of events costs the stream about
+// 10 us, which a measurement of whole steps should not pay at every launch.
+void timing_begin(const std::vector<std::string>& only = {}, int every = 1);
 std::map<std::string, std::pair<double, int64_t>> timing_collect();
 
 // RAII timer: accumulates into info[key] only when the key already exists (synchronous),

@@ -11,11 +11,14 @@ void MetaData::update_meta_data(int total_seq_len, int to_select_index_len, int 
     throw std::invalid_argument("update_meta_data: seq_len_info must be a prefix array starting at 0");
   if (int64_t(seq_len_info.back()) * RT_BLOCK != total_seq_len)
     throw std::invalid_argument("update_meta_data: total_seq_len does not match seq_len_info");
-  tensor_set->update_tensor_set(total_seq_len, to_select_index_len, to_select_index_position_len, seq_len_info);
-  semaphore->Signal(seq_len_info);
+  // the current micro-batch lane's set and pipeline (lane 0 unless the caller selected the other)
+  TensorSet::get_instance()->update_tensor_set(total_seq_len, to_select_index_len, to_select_index_position_len, seq_len_info);
+  Semaphore::get_instance()->Signal(seq_len_info);
 }
 
-void MetaData::terminate_thread() { semaphore->terminate(); }
+void MetaData::terminate_thread() {
+  for (int lane = 0; lane < LANES; ++lane) Semaphore::get_instance(lane)->terminate();
+}
 
 }  // namespace layers
 }  // namespace sparse_transformers

@@ -12,8 +12,8 @@ namespace layers {
 class MetaData {
  public:
   MetaData() {
-    tensor_set = TensorSet::get_instance();
-    semaphore = Semaphore::get_instance();
+    tensor_set = TensorSet::get_instance(0);
+    semaphore = Semaphore::get_instance(0);
   }
   // Resizes the scratch set, stores the geometry and wakes every layer's index worker.
   // The two length arguments are kept for signature compatibility; the CSR sizes are

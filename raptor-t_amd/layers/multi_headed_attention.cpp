@@ -28,15 +28,14 @@ MultiHeadedAttention::MultiHeadedAttention(torch::Tensor, torch::Tensor, torch::
   // both kept as [out, in]: the GEMMs are faster with both operands contiguous along the reduction
   qkv_weight_ = qkv_weight_.t().contiguous();
   dense_weight_ = dense_weight_.t().contiguous();
-  tensor_set = TensorSet::get_instance();
-  tensor_set->configure(d, qkv_weight_.scalar_type());
-  semaphore = Semaphore::get_instance();
-  semaphore->register_layer(layer_idx_, int(num_attention_heads), async);
-  handle_ = kernels::shared_gemm_handle();
+  for (int lane = 0; lane < LANES; ++lane) {        // every micro-batch lane knows every layer
+    TensorSet::get_instance(lane)->configure(d, qkv_weight_.scalar_type());
+    Semaphore::get_instance(lane)->register_layer(layer_idx_, int(num_attention_heads), async);
+  }
 }
 
 std::pair<std::vector<int>, std::vector<int>> MultiHeadedAttention::GenerateSparseBlockIndex() const {
-  const std::vector<int> sb = tensor_set->seq_len_info_;
+  const std::vector<int> sb = TensorSet::get_instance()->seq_len_info_;
   if (sb.size() < 2) throw std::runtime_error("GenerateSparseBlockIndex: no batch has been published");
   const int batch = int(sb.size()) - 1, heads = int(num_attention_heads_);
   int64_t n_idx = 0, n_pos = 0;
@@ -52,8 +51,9 @@ void MultiHeadedAttention::FuseGemm012AddBIasTranspose(const torch::Tensor& inpu
                                                        torch::Tensor& k_out, torch::Tensor& v_out,
                                                        torch::Tensor& seq_len_info_tensor, int total_seq_len, int d_num,
                                                        std::map<std::string, float>& info, bool kernel_fusion) const {
-  torch::Tensor tmp_qkv_out1 = tensor_set->get_tensor("tmp_qkv_out1");
-  kernels::MatMul(input_tensor, false, qkv_weight_, true, 1, tmp_qkv_out1, 0, handle_, "FuseGemm012AddBIasTranspose_MatMul");
+  torch::Tensor tmp_qkv_out1 = TensorSet::get_instance()->get_tensor("tmp_qkv_out1");
+  kernels::MatMul(input_tensor, false, qkv_weight_, true, 1, tmp_qkv_out1, 0, kernels::shared_gemm_handle(),
+                  "FuseGemm012AddBIasTranspose_MatMul");
   kernels::add_bias_and_transpose_kernel(qkv_bias_, tmp_qkv_out1, q_out, k_out, v_out, seq_len_info_tensor, batch_size_,
                                          head_num_, block_num_, head_size_, info, kernel_fusion);
 }
@@ -80,6 +80,10 @@ void MultiHeadedAttention::operator()(const torch::Tensor& input_tensor, const t
     throw std::invalid_argument("input/output must be [total tokens, hidden] for the published batch");
   if (seq_len_info_tensor.numel() != int64_t(seq_len_info.size()))
     throw std::invalid_argument("seq_len_info_tensor does not match seq_position_info");
+  // the scratch set, the index pipeline and the GEMM workspace of the current micro-batch lane
+  const TensorSet::Ptr tensor_set = TensorSet::get_instance();
+  const Semaphore::Ptr semaphore = Semaphore::get_instance();
+  rt_gemm_ctx* const handle_ = kernels::shared_gemm_handle();
   if (tensor_set->seq_len_info_ != seq_len_info)
     throw std::invalid_argument("the batch passed to the layer is not the one published by MetaData::update_meta_data");
 

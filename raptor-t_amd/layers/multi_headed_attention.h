@@ -53,9 +53,6 @@ class MultiHeadedAttention {
   float eps_;
   mutable int total_seq_len_ = 0, head_num_ = 0, d_num_ = 0, block_size_ = 0, head_size_ = 0, block_num_ = 0,
               batch_size_ = 0;
-  rt_gemm_ctx* handle_;
-  TensorSet::Ptr tensor_set;
-  Semaphore::Ptr semaphore;
 };
 
 }  // namespace layers

@@ -14,9 +14,9 @@ namespace py = pybind11;
 using namespace sparse_transformers;
 
 PYBIND11_MODULE(raptor_t, m) {
-  m.def("timing_begin", &layers::kernels::timing_begin, py::arg("only") = std::vector<std::string>(),
+  m.def("timing_begin", &layers::kernels::timing_begin, py::arg("only") = std::vector<std::string>(), py::arg("every") = 1,
         "Start bracketing kernel launchers with HIP events (no synchronisation): every launcher, or only the "
-        "named ones (each pair of events costs a few microseconds between kernels).");
+        "named ones, and of those only one call in `every` (each pair of events costs the stream about 10 us).");
   m.def("set_gemm_epilogue_fusion", &layers::kernels::set_gemm_epilogue_fusion,
         "BertIntermediate with kernel_fusion runs bias + GELU in the GEMM's epilogue (True, the default) or as the "
         "separate add_bias_act kernel (False).");
@@ -89,6 +89,12 @@ PYBIND11_MODULE(raptor_t, m) {
            py::arg("head_num"), py::arg("balanced") = false);
   }
 
+  m.def("set_micro_batch_lane", &layers::set_current_lane, py::arg("lane"),
+        "Selects which of the two independent sets of per-batch state (scratch tensors, published geometry, block-index "
+        "pipeline, GEMM workspace) the following calls use: a caller that keeps two micro-batches in flight on two "
+        "streams selects 0 or 1 before each call it makes for one of them.  Default 0.");
+  m.def("micro_batch_lane", &layers::current_lane);
+
   py::class_<layers::BertAttention>(m, "BertAttention")
       .def(py::init([](torch::Tensor& qkv_weight, torch::Tensor& qkv_bias, torch::Tensor& dense_weight,
                        torch::Tensor& dense_bias, torch::Tensor& layer_norm_weight, torch::Tensor& layer_norm_bias,
@@ -131,7 +137,7 @@ PYBIND11_MODULE(raptor_t, m) {
       }))
       .def("update_tensor_set", &layers::TensorSet::update_tensor_set)
       .def("get_tensor", &layers::TensorSet::get_tensor)
-      .def_static("get_instance", &layers::TensorSet::get_instance);
+      .def_static("get_instance", []() { return layers::TensorSet::get_instance(); });
 
   py::class_<layers::MetaData>(m, "MetaData")
       .def(py::init([]() { return new layers::MetaData(); }))
@@ -139,7 +145,8 @@ PYBIND11_MODULE(raptor_t, m) {
       .def("terminate_thread", &layers::MetaData::terminate_thread)
       .def_static("set_plan",
                   [](int plan_mode, int policy, int max_pos) {
-                    layers::Semaphore::get_instance()->set_plan(plan_mode, policy, max_pos);
+                    for (int lane = 0; lane < layers::LANES; ++lane)
+                      layers::Semaphore::get_instance(lane)->set_plan(plan_mode, policy, max_pos);
                   },
                   py::arg("plan_mode") = int(RT_PLAN_HF), py::arg("policy") = int(RT_POLICY_REFERENCE_PATCHED),
                   py::arg("max_pos") = 4096);

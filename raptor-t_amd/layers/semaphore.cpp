@@ -8,17 +8,20 @@
 namespace sparse_transformers {
 namespace layers {
 
-Semaphore::Ptr Semaphore::instance_ = nullptr;
+Semaphore::Ptr Semaphore::instance_[2];
 std::mutex Semaphore::instance_mutex_;
+static_assert(LANES == 2, "one Semaphore per micro-batch lane");
 
 static void check(int rc, const char* what) {
   if (rc != RT_OK) throw std::runtime_error(std::string(what) + ": " + rt_last_error_string());
 }
 
-Semaphore::Ptr Semaphore::get_instance() {
+Semaphore::Ptr Semaphore::get_instance() { return get_instance(current_lane()); }
+
+Semaphore::Ptr Semaphore::get_instance(int lane) {
   std::lock_guard<std::mutex> lk(instance_mutex_);
-  if (instance_ == nullptr) instance_ = Ptr(new Semaphore());
-  return instance_;
+  if (instance_[lane] == nullptr) instance_[lane] = Ptr(new Semaphore());
+  return instance_[lane];
 }
 
 Semaphore::~Semaphore() { rt_pipeline_destroy(pipeline_); }

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/raptor_t_hip.h"
+#include "tensor_set.h"
 
 namespace sparse_transformers {
 namespace layers {
@@ -35,7 +36,8 @@ class Semaphore {
   void terminate();
   // plan mode / policy / max positions used for the next pipeline that is created
   void set_plan(int plan_mode, int policy, int max_pos);
-  static Ptr get_instance();
+  static Ptr get_instance();            // the current micro-batch lane's (tensor_set.h)
+  static Ptr get_instance(int lane);
 
  private:
   Semaphore() {}
@@ -47,7 +49,7 @@ class Semaphore {
   bool pipeline_async_ = true, async_ = true;
   int plan_mode_ = RT_PLAN_HF, policy_ = RT_POLICY_REFERENCE_PATCHED, max_pos_ = 4096;
   std::vector<int> last_batch_;
-  static Ptr instance_;
+  static Ptr instance_[2];
   static std::mutex instance_mutex_;
 };
 

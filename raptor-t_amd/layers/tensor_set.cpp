@@ -5,8 +5,15 @@
 namespace sparse_transformers {
 namespace layers {
 
-TensorSet::Ptr TensorSet::instance_ = nullptr;
+TensorSet::Ptr TensorSet::instance_[LANES];
 std::mutex TensorSet::instance_mutex_;
+
+static int g_lane = 0;
+int current_lane() { return g_lane; }
+void set_current_lane(int lane) {
+  if (lane < 0 || lane >= LANES) throw std::invalid_argument("micro-batch lane must be 0 or 1");
+  g_lane = lane;
+}
 
 TensorSet::TensorSet(int64_t total_seq_len, int64_t to_select_index_len, int64_t to_select_index_position_len) {
   total_seq_len_ = int(total_seq_len);
@@ -59,10 +66,12 @@ torch::Tensor TensorSet::get_tensor(const std::string& tensor_name) {
   return it->second;
 }
 
-TensorSet::Ptr TensorSet::get_instance() {
+TensorSet::Ptr TensorSet::get_instance() { return get_instance(current_lane()); }
+
+TensorSet::Ptr TensorSet::get_instance(int lane) {
   std::lock_guard<std::mutex> lk(instance_mutex_);
-  if (instance_ == nullptr) instance_ = std::make_shared<TensorSet>(4096, 622, 65);   // tensor_set.h:61
-  return instance_;
+  if (instance_[lane] == nullptr) instance_[lane] = std::make_shared<TensorSet>(4096, 622, 65);   // tensor_set.h:61
+  return instance_[lane];
 }
 
 }  // namespace layers

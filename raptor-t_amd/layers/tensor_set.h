@@ -18,6 +18,16 @@
 namespace sparse_transformers {
 namespace layers {
 
+// Micro-batch lanes.  The process keeps LANES independent sets of the per-batch state (scratch tensors,
+// published geometry, block-index pipeline, GEMM workspace); get_instance() of TensorSet and Semaphore and
+// kernels::shared_gemm_handle() return the current lane's.  A caller that runs two micro-batches on two
+// streams selects the lane before every call it makes for one of them; everybody else stays on lane 0 and
+// sees the reference's single set.  The selection is a plain process-wide value: calls are issued from one
+// host thread.  No counterpart in the reference, which keeps one batch in flight.
+constexpr int LANES = 2;
+int current_lane();
+void set_current_lane(int lane);
+
 class TensorSet {
  public:
   typedef std::shared_ptr<TensorSet> Ptr;
@@ -35,7 +45,8 @@ class TensorSet {
                          std::vector<int> seq_len_info);
   // int32 device copy of seq_len_info_, refreshed by update_tensor_set
   torch::Tensor seq_len_info_device();
-  static Ptr get_instance();
+  static Ptr get_instance();            // the current lane's set
+  static Ptr get_instance(int lane);
 
  private:
   void allocate_locked();
@@ -44,7 +55,7 @@ class TensorSet {
   torch::Tensor seq_len_info_dev_;
   int64_t hidden_ = 768;
   torch::ScalarType dtype_ = torch::kHalf;
-  static Ptr instance_;
+  static Ptr instance_[LANES];
   static std::mutex instance_mutex_;
 };
 

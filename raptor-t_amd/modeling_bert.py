@@ -26,6 +26,7 @@ except ImportError as e:            # no silent fallback: the layer API is the p
     raise ImportError("the raptor_t extension is not built: run __graft_entry__.build() (%s)" % e)
 
 from . import capi, checkpoint
+from .util import generate_data_metainfo
 
 roctx = torch.cuda.nvtx             # torch maps these ranges onto roctx on ROCm
 
@@ -197,6 +198,61 @@ class BertEncoder:
                                          attention_output=attention_output, attention_mask=attention_mask,
                                          test_info=test_info, kernel_fusion=kernel_fusion,
                                          output_attentions=output_attentions, balanced=balanced)
+        return hidden_states, test_info
+
+    def call_two_streams(self, hidden_states, seq_lens, thread_block_limit, head_num, output_layer_temp,
+                         intermediate_temp, attention_output, test_info=None, kernel_fusion=True, balanced=True):
+        """The same forward pass with the batch cut in two micro-batches, each on a HIP stream of its own (equal
+        priority), so that one micro-batch's attention kernel runs beside the other's projection and FFN GEMMs
+        instead of between them.  The reference overlaps only the host's index generation with the GPU
+        (layers/multi_headed_attention.cpp:131-132, :179-185); its launches are serial on one stream.
+
+        `seq_lens`: token count of every sequence of the packed batch (multiples of 64).  The cut is the sequence
+        boundary nearest to half the tokens, so both micro-batches are row ranges of the caller's buffers and
+        nothing is copied.  The batch metadata of both halves is made here (cached per geometry) and published
+        on the two micro-batch lanes of the extension; the caller does not call MetaData.update_meta_data.
+        Returns when everything is queued; the caller's current stream waits for both streams."""
+        seq_lens = [int(n) for n in seq_lens]
+        key = (tuple(seq_lens), int(thread_block_limit), int(head_num))
+        if getattr(self, "_two_key", None) != key:
+            total, run, cut, best = sum(seq_lens), 0, 1, None
+            for i, n in enumerate(seq_lens[:-1]):
+                run += n
+                if best is None or abs(2 * run - total) < best:
+                    best, cut = abs(2 * run - total), i + 1
+            halves = [seq_lens] if len(seq_lens) < 2 else [seq_lens[:cut], seq_lens[cut:]]
+            self._two_parts, t0 = [], 0
+            for lens in halves:
+                info = generate_data_metainfo(lens, 64, thread_block_limit, head_num)
+                self._two_parts.append((slice(t0, t0 + sum(lens)), sum(lens), info))
+                t0 += sum(lens)
+            self._two_key = key
+        if not hasattr(self, "_two_streams"):
+            self._two_streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+            self._two_meta = cxx.MetaData()
+        test_info = {} if test_info is None else test_info
+        cur = torch.cuda.current_stream()
+        try:
+            for lane, (rows, t, (spi, spi_t, comp, ppi_t, pp_t)) in enumerate(self._two_parts):
+                cxx.set_micro_batch_lane(lane)
+                self._two_streams[lane].wait_stream(cur)
+                with torch.cuda.stream(self._two_streams[lane]):
+                    self._two_meta.update_meta_data(t, spi[-1] + 1, comp, spi)
+            for l in self.layer:                       # issue order: the two lanes' layers alternate
+                for lane, (rows, t, (spi, spi_t, comp, ppi_t, pp_t)) in enumerate(self._two_parts):
+                    cxx.set_micro_batch_lane(lane)
+                    with torch.cuda.stream(self._two_streams[lane]):
+                        _, test_info = l(hidden_states=hidden_states[rows], block_limit=thread_block_limit,
+                                         seq_position_info=spi, seq_position_info_tensor=spi_t,
+                                         partition_part_index_tensor=ppi_t, partition_part_tensor=pp_t,
+                                         output_layer_temp=output_layer_temp[rows],
+                                         intermediate_temp=intermediate_temp[rows],
+                                         attention_output=attention_output[rows], test_info=test_info,
+                                         kernel_fusion=kernel_fusion, balanced=balanced)
+        finally:
+            cxx.set_micro_batch_lane(0)
+        for lane in range(len(self._two_parts)):
+            cur.wait_stream(self._two_streams[lane])
         return hidden_states, test_info
 
     @staticmethod
