@@ -475,3 +475,51 @@ def test_padded_sequence_matches_huggingface_with_attention_mask(mb, ut, length,
     with pytest.raises((ValueError, RuntimeError)):
         model(p["input_ids"], length, 48, spi, spi_t, ppi_t, pp_t, attention_masks=mask.float(),
               token_type_ids=p["token_type_ids"], position_ids=p["position_ids"], intermediate_temp=inter)
+
+
+def test_padded_batch_of_several_sequences_matches_huggingface_per_sequence(mb, ut):
+    """A right-padded HuggingFace batch [B, L] whose sequences have different fills, packed by pack_padded_batch
+    (every sequence keeps its own length rounded up to 64) and run as one padding-free batch, against
+    HuggingFace BigBird run on each sequence alone at that length with its attention mask: two sparse
+    sequences (one with a single real token in its last block), one below twelve blocks (full attention in
+    both models) and a three-block one.  Compared on the real token rows."""
+    say("hf padded batch")
+    from transformers import BigBirdConfig, BigBirdModel
+    torch.manual_seed(5)
+    cfg = BigBirdConfig(vocab_size=1000, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        intermediate_size=256, max_position_embeddings=4096, attention_type="block_sparse",
+                        block_size=64, num_random_blocks=3, hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+    hf = BigBirdModel(cfg, add_pooling_layer=False).cuda().train()
+    with torch.no_grad():
+        for layer in hf.encoder.layer:
+            layer.attention.self.query.weight.mul_(6.0)
+            layer.attention.self.key.weight.mul_(6.0)
+            layer.attention.self.value.weight.mul_(5.0)
+    length, tokens = 1024, [1000, 700, 833, 130]
+    ids = torch.randint(1, 1000, (len(tokens), length), device="cuda")       # padding ids are not zero: a missed mask shows
+    mask = (torch.arange(length, device="cuda")[None, :] < torch.tensor(tokens, device="cuda")[:, None]).long()
+    p = ut.pack_padded_batch(ids, mask)
+    assert p["seq_lens"] == [1024, 704, 896, 192] and p["seq_tokens"] == tokens
+    model = mb.BertModelNoPooler.from_torch(hf, async_=True, dtype=torch.float16)
+    want = []
+    with torch.no_grad():
+        for s, (n, real) in enumerate(zip(p["seq_lens"], tokens)):
+            hf.set_attention_type("block_sparse")       # a short sequence switches the HuggingFace model to full attention for good
+            want.append(hf(input_ids=ids[s:s + 1, :n], attention_mask=mask[s:s + 1, :n]).last_hidden_state[0, :real].float().cpu())
+    t = sum(p["seq_lens"])
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(p["seq_lens"], 64, 48, 2)
+    meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+    inter = torch.empty(t, 256, dtype=torch.float16, device="cuda")
+    out, _ = model(p["input_ids"], t, 48, spi, spi_t, ppi_t, pp_t, attention_masks=p["seq_tokens_tensor"],
+                   token_type_ids=p["token_type_ids"], position_ids=p["position_ids"], intermediate_temp=inter)
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    got = ut.unpack_to_padded(out, p["seq_lens"], p["seq_tokens"], length)
+    assert got.shape == (len(tokens), length, 128)
+    for s, real in enumerate(tokens):
+        err = (got[s, :real].float().cpu() - want[s]).abs().max().item()
+        say("  sequence", s, "tokens", real, "err", err)
+        assert err <= 2e-2
+        assert bool((got[s, real:] == 0).all())
