@@ -634,3 +634,33 @@ def test_pipeline_on_device(capi):
             assert np.array_equal(got_idx.cpu().numpy(), want_idx) and np.array_equal(got_pos.cpu().numpy(), want_pos)
             pipe.release(layer)
     pipe.close()
+
+
+def test_attention_random_geometries(capi):
+    """Twenty seeded draws of batch geometry (1 to 7 sequences of 1 to 40 blocks, so sparse and full-attention
+    sequences mix), head count, dtype, plan mode, schedule (the kernel's own / a work plan of random size) and
+    padding, each against the oracle."""
+    say("attention random geometries")
+    rng = np.random.default_rng(2024)
+    for case in range(20):
+        batch = int(rng.integers(1, 8))
+        lens = [64 * int(rng.integers(1, 41)) for _ in range(batch)]
+        heads = int(rng.choice([1, 2, 3, 5]))
+        dtype = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
+        mode = capi.RT_PLAN_REFERENCE if rng.integers(0, 4) == 0 else None
+        n_wg = int(rng.integers(1, 60)) if rng.integers(0, 2) else 0
+        padded = bool(rng.integers(0, 2))
+        seq_tokens = [n - int(rng.integers(0, 64)) for n in lens] if padded else None
+        say("  case", case, lens, heads, dtype, mode, n_wg, seq_tokens)
+        t = sum(lens)
+        g = torch.Generator().manual_seed(1000 + case)
+        q, k, v = (torch.randn(t, heads, 64, generator=g).to(dtype).cuda() for _ in range(3))
+        out, ref = lh.run_attention(capi, q, k, v, lens, heads, seed=case, mode=mode, n_wg=n_wg, seq_tokens=seq_tokens)
+        rows = torch.ones(t, dtype=torch.bool)
+        if padded:                                         # padded query rows are computed but not specified
+            start = 0
+            for n, real in zip(lens, seq_tokens):
+                rows[start + real:start + n] = False
+                start += n
+        assert torch.isfinite(out.float()).all(), case
+        assert lh.excess(out[rows.cuda()], ref[rows], dtype, k=1.0) <= 0, case

@@ -109,3 +109,23 @@ def test_sequence_pool_and_pooler_match_torch_and_hand_cases():
     assert (got - want).abs().max().item() <= 1e-6
     one = ol.pooler(torch.tensor([[1.0, 2.0]]), torch.tensor([[0.5], [0.25]]), torch.tensor([-1.0]))
     assert abs(one.item() - 0.0) < 1e-7                       # tanh(0.5 + 0.5 - 1)
+
+
+def test_stored_tensors_option_rounds_between_kernels_only():
+    """encoder_layer(store_dtype=...) rounds every tensor that passes from one kernel to the next and nothing else:
+    with fp32 as the storage type it is the plain layer, with bf16 the output is a bf16 value everywhere and stays
+    within a few bf16 ulp of the plain layer."""
+    from oracle import metadata as md
+    g = torch.Generator().manual_seed(0)
+    hidden, heads, ffn, lens = 128, 2, 256, [832, 128]
+    w = ol.random_layer_weights(hidden, ffn, g)
+    x = torch.randn(sum(lens), hidden, generator=g)
+    sb = md.seq_prefix_blocks(lens)
+    idx, pos = md.hf_to_index(lens, 0, heads)
+    plain = ol.encoder_layer(x, w, heads, sb, idx, pos, heads)
+    same = ol.encoder_layer(x, w, heads, sb, idx, pos, heads, store_dtype=torch.float32)
+    assert torch.equal(plain, same)
+    rounded = ol.encoder_layer(x, w, heads, sb, idx, pos, heads, store_dtype=torch.bfloat16)
+    assert torch.equal(rounded, rounded.to(torch.bfloat16).float())
+    err = (rounded - plain).abs().max().item()
+    assert 0 < err <= 0.1, err
