@@ -220,9 +220,9 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    # Timed region: of the attention launches (the kernel the roofline object is about) one in five is bracketed
-    # with events, rotating through the layers; a pair of events costs the stream about 18 us (5 % of the step if
-    # every attention launch carried one, 10 % with every launcher).
+    # Timed region: of the attention launches (the kernel the roofline object is about) one in five carries a pair
+    # of events that take the dispatch's own start and end, rotating through the layers; a timed launch costs the
+    # stream about 5 us (0.6 % of the step if every attention launch carried one).
     mb.cxx.timing_begin(["attention"], 5)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -309,8 +309,9 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
         "two_streams": two_streams,
         "kernel_us_per_launch": per,
         "kernel_us_per_step": {k: v[0] / args.steps for k, v in timing_all.items()},
-        "kernel_timing": "attention: HIP events around one launch in five inside the timed steps; the others: a second "
-                         "pass over the same steps with every launcher bracketed",
+        "kernel_timing": "HIP events holding each dispatch's own start and end (hipExtLaunchKernelGGL; the vendor GEMMs: "
+                         "events recorded around the call).  attention: one launch in five inside the timed steps; "
+                         "the others: a second pass over the same steps with every launcher timed",
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(seq_lens, hidden, heads, ffn, layers, args.cpu_sample_seqs)
@@ -318,12 +319,16 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
 
 
 def time_kernel(fn, steps, warmup, settle_ms=25.0):
-    """Median GPU duration of one launch in microseconds.  After the warm-up launches the kernel keeps running
-    for `settle_ms`: from idle the GPU takes some tens of launches to reach its sustained clocks (the first
-    launches of a 100 us kernel measure 10-15 % slow), and a kernel inside a running job never sees that ramp.
-    The timed launches are queued behind a spin kernel that keeps the GPU busy while the host enqueues all of
-    them: a launch through Python costs the host about 10 us, more than a small kernel runs, and an idle GPU
-    waiting for its next launch would be timed as part of it."""
+    """Median GPU duration of one launch in microseconds; `fn` launches exactly one kernel of the library.  The
+    duration is the dispatch's own (capi.time_next_launch: the start and end the GPU stamps on the kernel, what
+    rocprofv3 reports), on the stream `fn` launches on; a pair of recorded events around a launch would add the
+    gaps to its neighbours, 2-5 us here.  After the warm-up launches the kernel keeps running for `settle_ms`:
+    from idle the GPU takes some tens of launches to reach its sustained clocks (the first launches of a 100 us
+    kernel measure 10-15 % slow), and a kernel inside a running job never sees that ramp.  The timed launches are
+    queued behind a spin kernel that keeps the GPU busy while the host enqueues all of them, so that they run back
+    to back as in a job (a launch through Python costs the host about 10 us, more than a small kernel runs)."""
+    pkg = graft.load_package()
+    cxx = importlib.import_module("raptor_t_amd.modeling_bert").cxx
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -336,14 +341,13 @@ def time_kernel(fn, steps, warmup, settle_ms=25.0):
     fn()
     host_us = (time.perf_counter() - t0) * 1e6                 # what one enqueue costs the host
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    evs = [cxx.event_pair_create() for _ in range(steps)]
     torch.cuda._sleep(int(2.4e3 * (3.0 * host_us + 20.0) * steps))   # cycles: three times the host's enqueue time
     for a, b in evs:
-        a.record()
+        pkg.capi.time_next_launch(a, b)
         fn()
-        b.record()
     torch.cuda.synchronize()
-    return float(np.median([a.elapsed_time(b) for a, b in evs])) * 1e3      # microseconds
+    return float(np.median([cxx.event_pair_elapsed_us(a, b) for a, b in evs]))
 
 
 def run_attention_only(args):

@@ -69,6 +69,18 @@ enum { RT_POLICY_REFERENCE_PATCHED = 0, RT_POLICY_HF_UPSTREAM = 1 };
 const char* rt_last_error_string(void);
 int rt_abi_version(void);
 
+/* Timing of one kernel by its own dispatch.  The reference times a launcher with the host clock around the
+ * launch (layers/kernels/add_bias_act.cu:109-131, the `info` map of every launcher); a pair of events recorded
+ * around a launch also counts the gaps to the neighbouring kernels.  After this call the next kernel that one
+ * of this library's kernel entry points (every one below except the vendor GEMMs; each launches one kernel,
+ * rt_bs_attention_fwd_no_alloc a small clearing kernel before it that does not count) launches from the calling
+ * thread writes the start and end timestamps of its dispatch into the two hipEvent_t (created by the caller,
+ * either may be NULL); hipEventElapsedTime between them is the kernel's duration as a profiler reports it.
+ * One launch consumes the pair; (NULL, NULL) withdraws a pair no launch has taken.  Returns 1 if the call
+ * replaced or withdrew a pair that was still waiting for a launch, 0 otherwise.  Not for use while a stream
+ * is being captured into a graph. */
+int rt_time_next_launch(void* start_event, void* stop_event);
+
 /* ------------------------------------------------------------------ host metadata */
 
 /* numpy.random.seed(seed) followed by `count` calls of numpy.random.permutation(n_i):

@@ -20,7 +20,7 @@ RT_EPILOGUE_NONE, RT_EPILOGUE_BIAS, RT_EPILOGUE_BIAS_GELU = 0, 1, 2
 RT_GEMM_TUNE_ALL = -1
 
 EXPORTS = [
-    "rt_last_error_string", "rt_abi_version", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
+    "rt_last_error_string", "rt_abi_version", "rt_time_next_launch", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_meta_check_partition", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows", "rt_bs_attention_fwd_no_alloc",
@@ -50,6 +50,7 @@ def lib():
         L.rt_last_error_string.restype = ctypes.c_char_p
         i32p, i64p, vp = ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64), ctypes.c_void_p
         I, U, L64, F = ctypes.c_int, ctypes.c_uint32, ctypes.c_int64, ctypes.c_float
+        L.rt_time_next_launch.argtypes = [vp, vp]
         L.rt_meta_np_permutations.argtypes = [U, i32p, I, i32p]
         L.rt_meta_seq_prefix_blocks.argtypes = [i32p, I, i32p]
         L.rt_meta_rand_attn.argtypes = [I, U, I, I, I, i32p]
@@ -296,6 +297,13 @@ def bias_gelu(out, bias):
     rows, width = out.shape
     check(lib().rt_bias_gelu(_dp(out, name="out"), _dp(bias, out.dtype, width, "bias"), rows, width, _dtype_code(out),
                              _stream()))
+
+
+def time_next_launch(start_event, stop_event):
+    """Hands two hipEvent_t (integers / c_void_p; None = NULL) to the calling thread's next kernel launch of the
+    library, which writes its dispatch's start and end into them.  (None, None) withdraws a waiting pair.
+    Returns 1 if a pair was still waiting for a launch."""
+    return lib().rt_time_next_launch(start_event, stop_event)
 
 
 RT_POOL_FIRST, RT_POOL_LAST, RT_POOL_MEAN, RT_POOL_MAX = 0, 1, 2, 3

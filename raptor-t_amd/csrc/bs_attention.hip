@@ -52,7 +52,7 @@
 #include <mutex>
 #include <type_traits>
 
-#include "rt_common.h"
+#include "rt_launch.h"
 
 
 namespace {
@@ -1211,14 +1211,14 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
     Args<_Float16> a{(const _Float16*)q, (const _Float16*)k, (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch,
                      heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
                      (const _Float16*)q_rows, (const _Float16*)q_bias, q_scale, queues, queues_clear};
-    if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<_Float16, true>), dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((bs_attention_kernel<_Float16, false>), dim3(grid), dim3(256), 0, st, a);
+    if (seq_tokens_dev) RT_LAUNCH((bs_attention_kernel<_Float16, true>), dim3(grid), dim3(256), 0, st, a);
+    else RT_LAUNCH((bs_attention_kernel<_Float16, false>), dim3(grid), dim3(256), 0, st, a);
   } else {
     Args<__bf16> a{(const __bf16*)q, (const __bf16*)k, (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads,
                    total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
                    (const __bf16*)q_rows, (const __bf16*)q_bias, q_scale, queues, queues_clear};
-    if (seq_tokens_dev) hipLaunchKernelGGL((bs_attention_kernel<__bf16, true>), dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((bs_attention_kernel<__bf16, false>), dim3(grid), dim3(256), 0, st, a);
+    if (seq_tokens_dev) RT_LAUNCH((bs_attention_kernel<__bf16, true>), dim3(grid), dim3(256), 0, st, a);
+    else RT_LAUNCH((bs_attention_kernel<__bf16, false>), dim3(grid), dim3(256), 0, st, a);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "bs_attention launch failed: %s", hipGetErrorString(e));

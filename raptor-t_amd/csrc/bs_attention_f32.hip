@@ -20,7 +20,7 @@
 
 #include <cstdint>
 
-#include "rt_common.h"
+#include "rt_launch.h"
 
 namespace {
 
@@ -209,8 +209,8 @@ int launch_attention_f32(const void* q, const void* q_rows, const void* q_bias, 
                   (const float*)q_rows, (const float*)q_bias, q_scale};
   const unsigned grid = from_idx ? unsigned(n_wg) : unsigned(total_blocks) * unsigned(heads);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (seq_tokens_dev) hipLaunchKernelGGL(bs_attention_f32_kernel<true>, dim3(grid), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(bs_attention_f32_kernel<false>, dim3(grid), dim3(256), 0, st, a);
+  if (seq_tokens_dev) RT_LAUNCH(bs_attention_f32_kernel<true>, dim3(grid), dim3(256), 0, st, a);
+  else RT_LAUNCH(bs_attention_f32_kernel<false>, dim3(grid), dim3(256), 0, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "fp32 bs_attention launch failed: %s", hipGetErrorString(e));
   return RT_OK;

@@ -15,7 +15,7 @@
 
 #include <type_traits>
 
-#include "rt_common.h"
+#include "rt_launch.h"
 
 namespace {
 
@@ -172,7 +172,7 @@ void launch_ln(T* out, const T* res, const T* bias, const T* gamma, const T* bet
                hipStream_t st) {
   const int rows_per_wg = 256 / G;
   const unsigned grid = unsigned((rows + rows_per_wg - 1) / rows_per_wg);
-  hipLaunchKernelGGL((bias_residual_layernorm_kernel<T, CHUNKS, G>), dim3(grid), dim3(256), 0, st, out, res, bias,
+  RT_LAUNCH((bias_residual_layernorm_kernel<T, CHUNKS, G>), dim3(grid), dim3(256), 0, st, out, res, bias,
                      gamma, beta, rows, eps);
 }
 
@@ -198,7 +198,7 @@ int ln_dispatch(void* out, const void* res, const void* bias, const void* gamma,
     }
   }
   const unsigned grid = unsigned((rows + 3) / 4);
-  hipLaunchKernelGGL((bias_residual_layernorm_generic_kernel<T>), dim3(grid), dim3(256), 0, st, o, r, b, g, be, rows,
+  RT_LAUNCH((bias_residual_layernorm_generic_kernel<T>), dim3(grid), dim3(256), 0, st, o, r, b, g, be, rows,
                      hidden, eps);
   return RT_OK;
 }
@@ -317,7 +317,7 @@ template <typename TT, typename TO, int CHUNKS, int G>
 void launch_embed(const EmbedArgs<TT, TO>& a, hipStream_t st) {
   const int rows_per_wg = 256 / G;
   const unsigned grid = unsigned((a.rows + rows_per_wg - 1) / rows_per_wg);
-  hipLaunchKernelGGL((embed_layernorm_kernel<TT, TO, CHUNKS, G>), dim3(grid), dim3(256), 0, st, a);
+  RT_LAUNCH((embed_layernorm_kernel<TT, TO, CHUNKS, G>), dim3(grid), dim3(256), 0, st, a);
 }
 
 template <typename TT, typename TO>
@@ -334,7 +334,7 @@ void embed_dispatch(const EmbedArgs<TT, TO>& a, int hidden, hipStream_t st) {
     }
   }
   const unsigned grid = unsigned((a.rows + 3) / 4);
-  hipLaunchKernelGGL((embed_layernorm_generic_kernel<TT, TO>), dim3(grid), dim3(256), 0, st, a, hidden);
+  RT_LAUNCH((embed_layernorm_generic_kernel<TT, TO>), dim3(grid), dim3(256), 0, st, a, hidden);
 }
 
 template <typename TT>
@@ -633,11 +633,11 @@ int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype
   const unsigned grid = unsigned(want);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == RT_F16)
-    hipLaunchKernelGGL(bias_gelu_kernel<__half>, dim3(grid), dim3(256), 0, st, (__half*)out, (const __half*)bias, n_vec, width / n);
+    RT_LAUNCH(bias_gelu_kernel<__half>, dim3(grid), dim3(256), 0, st, (__half*)out, (const __half*)bias, n_vec, width / n);
   else if (dtype == RT_BF16)
-    hipLaunchKernelGGL(bias_gelu_kernel<__hip_bfloat16>, dim3(grid), dim3(256), 0, st, (__hip_bfloat16*)out, (const __hip_bfloat16*)bias, n_vec, width / n);
+    RT_LAUNCH(bias_gelu_kernel<__hip_bfloat16>, dim3(grid), dim3(256), 0, st, (__hip_bfloat16*)out, (const __hip_bfloat16*)bias, n_vec, width / n);
   else
-    hipLaunchKernelGGL(bias_gelu_kernel<float>, dim3(grid), dim3(256), 0, st, (float*)out, (const float*)bias, n_vec, width / n);
+    RT_LAUNCH(bias_gelu_kernel<float>, dim3(grid), dim3(256), 0, st, (float*)out, (const float*)bias, n_vec, width / n);
   return check_launch("bias_gelu");
 }
 
@@ -654,10 +654,10 @@ int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void*
   auto launch = [&](auto tag) {
     typedef decltype(tag) T;
     if (q)
-      hipLaunchKernelGGL((qkv_bias_split_kernel<T, true>), grid, dim3(256), 0, st, (const T*)qkv, (const T*)bias, (T*)q,
+      RT_LAUNCH((qkv_bias_split_kernel<T, true>), grid, dim3(256), 0, st, (const T*)qkv, (const T*)bias, (T*)q,
                          (T*)k, (T*)vt, seq_blocks_dev, batch, heads, q_scale);
     else
-      hipLaunchKernelGGL((qkv_bias_split_kernel<T, false>), grid, dim3(256), 0, st, (const T*)qkv, (const T*)bias,
+      RT_LAUNCH((qkv_bias_split_kernel<T, false>), grid, dim3(256), 0, st, (const T*)qkv, (const T*)bias,
                          (T*)nullptr, (T*)k, (T*)vt, seq_blocks_dev, batch, heads, q_scale);
   };
   if (dtype == RT_F16) launch(__half());
@@ -675,11 +675,11 @@ int rt_unpack_head_tiles(const void* packed, void* dst, const int* seq_blocks_de
   dim3 grid(total_blocks, heads);
   const int tr = transposed ? 1 : 0;
   if (dtype == RT_F16)
-    hipLaunchKernelGGL(unpack_head_tiles_kernel<__half>, grid, dim3(256), 0, st, (const __half*)packed, (__half*)dst, seq_blocks_dev, batch, heads, tr);
+    RT_LAUNCH(unpack_head_tiles_kernel<__half>, grid, dim3(256), 0, st, (const __half*)packed, (__half*)dst, seq_blocks_dev, batch, heads, tr);
   else if (dtype == RT_BF16)
-    hipLaunchKernelGGL(unpack_head_tiles_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)packed, (__hip_bfloat16*)dst, seq_blocks_dev, batch, heads, tr);
+    RT_LAUNCH(unpack_head_tiles_kernel<__hip_bfloat16>, grid, dim3(256), 0, st, (const __hip_bfloat16*)packed, (__hip_bfloat16*)dst, seq_blocks_dev, batch, heads, tr);
   else if (dtype == RT_F32)
-    hipLaunchKernelGGL(unpack_head_tiles_kernel<float>, grid, dim3(256), 0, st, (const float*)packed, (float*)dst, seq_blocks_dev, batch, heads, tr);
+    RT_LAUNCH(unpack_head_tiles_kernel<float>, grid, dim3(256), 0, st, (const float*)packed, (float*)dst, seq_blocks_dev, batch, heads, tr);
   else
     return rt::fail(RT_EINVAL, "unknown dtype %d", dtype);
   return check_launch("unpack_head_tiles");
@@ -729,7 +729,7 @@ int rt_sequence_pool(const void* hidden, const int* seq_blocks_dev, const int* s
   auto launch = [&](auto tag) {
     typedef decltype(tag) T;
     const int per_wg = 8 * Vec<T>::N;
-    hipLaunchKernelGGL(sequence_pool_kernel<T>, dim3(batch, (width + per_wg - 1) / per_wg), dim3(256), 0, st,
+    RT_LAUNCH(sequence_pool_kernel<T>, dim3(batch, (width + per_wg - 1) / per_wg), dim3(256), 0, st,
                        (const T*)hidden, seq_blocks_dev, seq_tokens_dev, width, mode, (T*)out);
   };
   if (dtype == RT_F16) launch(__half());
@@ -748,7 +748,7 @@ int rt_pooler_dense_tanh(const void* pooled, const void* weight_t, const void* b
   hipStream_t st = static_cast<hipStream_t>(stream);
   auto launch = [&](auto tag) {
     typedef decltype(tag) T;
-    hipLaunchKernelGGL(pooler_dense_tanh_kernel<T>, dim3((d_out + 3) / 4), dim3(256), 0, st, (const T*)pooled,
+    RT_LAUNCH(pooler_dense_tanh_kernel<T>, dim3((d_out + 3) / 4), dim3(256), 0, st, (const T*)pooled,
                        (const T*)weight_t, (const T*)bias, (T*)out, batch, d_in, d_out);
   };
   if (dtype == RT_F16) launch(__half());

@@ -25,6 +25,14 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+static thread_local LaunchEvents g_launch_events = {nullptr, nullptr};
+LaunchEvents take_launch_events() {
+  const LaunchEvents ev = g_launch_events;
+  g_launch_events = LaunchEvents{nullptr, nullptr};
+  return ev;
+}
+static void set_launch_events(void* start, void* stop) { g_launch_events = LaunchEvents{start, stop}; }
+
 // numpy's legacy generator: MT19937 seeded by init_genrand, 32-bit tempered draws,
 // bounded integers by masked rejection, Fisher-Yates from the top (numpy
 // RandomState.seed / .permutation).
@@ -225,6 +233,11 @@ using namespace rt;
 extern "C" {
 
 const char* rt_last_error_string(void) { return error_buffer(); }
+int rt_time_next_launch(void* start_event, void* stop_event) {
+  const rt::LaunchEvents pending = rt::take_launch_events();
+  rt::set_launch_events(start_event, stop_event);
+  return (pending.start || pending.stop) ? 1 : 0;
+}
 int rt_abi_version(void) { return 1; }
 
 int rt_meta_np_permutations(uint32_t seed, const int* n, int count, int* out) {

@@ -10,6 +10,11 @@ namespace rt {
 char* error_buffer();                       // per-thread, 512 bytes
 int fail(int code, const char* fmt, ...);   // formats into the buffer, returns code
 
+// The pair of events rt_time_next_launch left for this thread's next kernel launch (both null: none); taking
+// them clears them.
+struct LaunchEvents { void* start; void* stop; };
+LaunchEvents take_launch_events();
+
 // Block-sparse attention with every tensor in fp32 (bs_attention_f32.hip); arguments as the fp16 / bf16 launch,
 // already checked by it.
 int launch_attention_f32(const void* q, const void* q_rows, const void* q_bias, float q_scale, const void* k,

@@ -130,7 +130,8 @@ std::map<std::string, std::pair<double, int64_t>> timing_collect() {
   return out;
 }
 
-ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* key) : key_(key) {
+ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* key, bool own_dispatch)
+    : key_(key), own_dispatch_(own_dispatch) {
   auto it = info.find(key);
   if (it != info.end()) slot_ = &it->second;
   {
@@ -144,13 +145,22 @@ ScopedGpuTimer::ScopedGpuTimer(std::map<std::string, float>& info, const char* k
   if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) { slot_ = nullptr; deferred_ = false; return; }
   start_ = a;
   stop_ = b;
-  (void)hipEventRecord(a, static_cast<hipStream_t>(current_stream()));
+  if (own_dispatch_) (void)rt_time_next_launch(a, b);
+  else (void)hipEventRecord(a, static_cast<hipStream_t>(current_stream()));
 }
 
 ScopedGpuTimer::~ScopedGpuTimer() {
   if (!slot_ && !deferred_) return;
   hipEvent_t a = static_cast<hipEvent_t>(start_), b = static_cast<hipEvent_t>(stop_);
-  (void)hipEventRecord(b, static_cast<hipStream_t>(current_stream()));
+  if (own_dispatch_) {
+    if (rt_time_next_launch(nullptr, nullptr) == 1) {      // no kernel took the pair: nothing was measured
+      (void)hipEventDestroy(a);
+      (void)hipEventDestroy(b);
+      return;
+    }
+  } else {
+    (void)hipEventRecord(b, static_cast<hipStream_t>(current_stream()));
+  }
   if (slot_) {
     (void)hipEventSynchronize(b);
     float ms = 0.f;
@@ -267,7 +277,7 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
     require_data(v, "v", dt, per_tensor);
     require_index(seq_len_info_tensor, "seq_len_info_tensor", int64_t(batch_size) + 1);
   }
-  ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel");
+  ScopedGpuTimer timer(info, "add_bias_and_transpose_kernel", kernel_fusion);
   // the attention kernel evaluates the softmax in base 2: fold log2(e) into the Q scale
   const float scale = kQScale;
   if (kernel_fusion) {
@@ -325,7 +335,7 @@ void add_bias_and_layernorm_kernel(torch::Tensor& out, const torch::Tensor& inpu
     require_data(layernorm_weight, "layernorm weight", dt, normalized_len);
     require_data(layernorm_bias, "layernorm bias", dt, normalized_len);
   }
-  ScopedGpuTimer timer(info, "add_bias_and_layernorm_kernel");
+  ScopedGpuTimer timer(info, "add_bias_and_layernorm_kernel", kernel_fusion);
   if (kernel_fusion) {
     check(rt_bias_residual_layernorm(out.data_ptr(), input_data.data_ptr(), bias.data_ptr(),
                                      layernorm_weight.data_ptr(), layernorm_bias.data_ptr(), seq_len, normalized_len,
@@ -345,7 +355,7 @@ void add_bias_act_kernel(const torch::Tensor& bias, torch::Tensor& out, int tota
     throw std::invalid_argument("add_bias_act_kernel: out holds " + std::to_string(out.numel()) +
                                 " elements, total_seq_len x dim_size is " + std::to_string(int64_t(total_seq_len) * dim_size));
   require_data(bias, "bias", out.scalar_type(), dim_size);
-  ScopedGpuTimer timer(info, "add_bias_act_kernel");
+  ScopedGpuTimer timer(info, "add_bias_act_kernel", kernel_fusion);
   if (kernel_fusion) {
     check(rt_bias_gelu(out.data_ptr(), bias.data_ptr(), total_seq_len, dim_size, dtype_code(out), current_stream()),
           "rt_bias_gelu");
@@ -374,7 +384,7 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
   require_data(k, "k", out.scalar_type(), per_tensor);
   require_data(v, "v", out.scalar_type(), per_tensor);
   require_index(seq_len_info_tensor, "seq_len_info_tensor", int64_t(batch_size) + 1);
-  ScopedGpuTimer timer(info, "attention");
+  ScopedGpuTimer timer(info, "attention", true);
   const int* tokens = nullptr;
   if (seq_tokens.defined() && seq_tokens.numel() > 0) {
     if (!seq_tokens.is_cuda() || !seq_tokens.is_contiguous() || seq_tokens.scalar_type() != torch::kInt32 ||

@@ -35,16 +35,19 @@ rt_gemm_ctx* shared_gemm_handle();
 // synchronising; timing_collect() synchronises once and returns, per launcher name,
 // (total microseconds, number of launches).  Lets a harness time kernels inside an
 // otherwise free-running loop.
-// `every` > 1 brackets only one in `every` calls of each launcher: a pair of events costs the stream about
-// 10 us, which a measurement of whole steps should not pay at every launch.
+// `every` > 1 times only one in `every` calls of each launcher: a pair of events costs the stream 5 to 10 us,
+// which a measurement of whole steps should not pay at every launch.
 void timing_begin(const std::vector<std::string>& only = {}, int every = 1);
 std::map<std::string, std::pair<double, int64_t>> timing_collect();
 
 // RAII timer: accumulates into info[key] only when the key already exists (synchronous),
-// and feeds the deferred timing when it is active.
+// and feeds the deferred timing when it is active.  `own_dispatch`: the launcher starts exactly one kernel of
+// the library; its events then carry the dispatch's own start and end (rt_time_next_launch), the duration a
+// profiler reports.  Otherwise (vendor GEMMs) the events are recorded on the stream before and after the call
+// and also count the gaps to the neighbouring kernels.
 class ScopedGpuTimer {
  public:
-  ScopedGpuTimer(std::map<std::string, float>& info, const char* key);
+  ScopedGpuTimer(std::map<std::string, float>& info, const char* key, bool own_dispatch = false);
   ~ScopedGpuTimer();
 
  private:
@@ -53,6 +56,7 @@ class ScopedGpuTimer {
   const char* key_ = nullptr;
   void* start_ = nullptr;
   void* stop_ = nullptr;
+  bool own_dispatch_ = false;
 };
 
 // kernels::MatMul (layers/kernels/mat_mul.cpp:9-96): out[M,N] = A[M,K] . B[K,N], or

@@ -4,6 +4,9 @@
 // hard-codes (LayerNorm eps); `set_plan` selects the random-block plan generator.
 #include <pybind11/stl.h>
 #include <torch/extension.h>
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
 
 #include "bert_attention.h"
 #include "bert_intermediate.h"
@@ -40,6 +43,23 @@ PYBIND11_MODULE(raptor_t, m) {
   m.def("attention_q_from_rows", &layers::kernels::attention_q_from_rows);
   m.def("timing_collect", &layers::kernels::timing_collect,
         "Synchronise and return {launcher: (total microseconds, launches)} since timing_begin().");
+  m.def("event_pair_create", []() {
+          hipEvent_t a = nullptr, b = nullptr;
+          if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) throw std::runtime_error("hipEventCreate failed");
+          return std::make_pair(reinterpret_cast<std::uintptr_t>(a), reinterpret_cast<std::uintptr_t>(b));
+        },
+        "Two hipEvent_t as integers, for rt_time_next_launch (capi.time_next_launch) of a caller that drives the C "
+        "ABI itself; event_pair_elapsed_us ends their life.");
+  m.def("event_pair_elapsed_us", [](std::uintptr_t a, std::uintptr_t b) {
+          hipEvent_t ea = reinterpret_cast<hipEvent_t>(a), eb = reinterpret_cast<hipEvent_t>(b);
+          float ms = -1.0f;
+          const bool ok = hipEventSynchronize(eb) == hipSuccess && hipEventElapsedTime(&ms, ea, eb) == hipSuccess;
+          (void)hipEventDestroy(ea);
+          (void)hipEventDestroy(eb);
+          if (!ok) throw std::runtime_error("the events were never given to a launch, or the launch failed");
+          return double(ms) * 1000.0;
+        },
+        "Waits for the stop event, returns the microseconds between the two and destroys both.");
   // The tensor-level launchers the layer objects call, under the reference's names (layers/kernels/kernel.h):
   // for callers that drive single kernels, and so that their argument checks can be exercised without a GPU.
   {

@@ -124,6 +124,21 @@ def test_error_paths_return_codes_not_exits(capi):
                                                  ctypes.c_void_p(16), ctypes.c_void_p(16), 4, 7, 1e-5, 0, None) == capi.RT_EINVAL
 
 
+def test_launch_event_pair_is_per_thread_and_withdrawable(capi):
+    """rt_time_next_launch only stores the pair (no GPU call): a second call reports the pair that no launch took,
+    and another thread neither sees nor disturbs it."""
+    import threading
+    assert capi.time_next_launch(None, None) == 0
+    assert capi.time_next_launch(ctypes.c_void_p(8), ctypes.c_void_p(16)) == 0
+    seen = []
+    th = threading.Thread(target=lambda: seen.append(capi.time_next_launch(None, None)))
+    th.start()
+    th.join()
+    assert seen == [0]
+    assert capi.time_next_launch(None, None) == 1          # still there: withdrawn now
+    assert capi.time_next_launch(None, None) == 0
+
+
 def _host_csr(ptr, n):
     return np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_int)), shape=(n,)).copy()
 

@@ -230,6 +230,34 @@ def test_fused_and_unfused_paths_agree(mb, ut):
     assert (outs[0] - outs[2]).abs().max().item() <= 2e-2
 
 
+def test_dispatch_events_time_exactly_one_launch(pkg, mb):
+    """rt_time_next_launch: the next kernel of the library writes its own start and end into the caller's events;
+    the launch after it is an ordinary one, and a pair no launch took cannot be read."""
+    say("dispatch events")
+    capi = pkg.capi
+    rows, width = 4096, 768
+    g = torch.Generator().manual_seed(3)
+    x, res = (torch.randn(rows, width, generator=g).half().cuda() for _ in range(2))
+    bias, gamma, beta = (torch.randn(width, generator=g).half().cuda() for _ in range(3))
+    out = x.clone()
+    capi.bias_residual_layernorm(out, res, bias, gamma, beta, 1e-5)          # first launch: module load
+    torch.cuda.synchronize()
+    a, b = mb.cxx.event_pair_create()
+    assert capi.time_next_launch(a, b) == 0
+    out.copy_(x)
+    capi.bias_residual_layernorm(out, res, bias, gamma, beta, 1e-5)
+    assert capi.time_next_launch(None, None) == 0                            # the launch took the pair
+    first = out.clone()
+    out.copy_(x)
+    capi.bias_residual_layernorm(out, res, bias, gamma, beta, 1e-5)          # an ordinary launch again
+    us = mb.cxx.event_pair_elapsed_us(a, b)
+    assert 0.5 < us < 2000.0, us
+    assert torch.equal(out, first)
+    c, d = mb.cxx.event_pair_create()
+    with pytest.raises(RuntimeError):
+        mb.cxx.event_pair_elapsed_us(c, d)
+
+
 def test_batches_of_changing_geometry_back_to_back(mb, ut):
     """Eight batches of different geometry enqueued without a synchronisation in between (the index workers run
     ahead, the slots of the block-index pipeline are reused every second batch): every batch matches the oracle."""
