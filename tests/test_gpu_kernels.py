@@ -324,6 +324,39 @@ def test_attention_reference_plan_shared_heads(capi):
     assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
 
 
+def test_attention_on_the_reference_test_case(capi):
+    """The one attention test the reference itself runs (layers/test.cpp:78-242): a single 4096-token sequence,
+    12 heads, Q = K = V = the ramp 6/4095 * (i % 4096) - 2 over the head-major [12][64][64][64] buffer (:11-16,
+    :182-196), its hard-coded block index shared by all heads (:89-91) and its 160-CTA partition (:95-164), which
+    the kernel walks here.  The reference compares its fp16 kernel with its fp32 one at 0.1 (:35-48); the oracle
+    is held to this build's 2e-2.  Scores reach 1000, so every row takes the moving-maximum route."""
+    import json, os
+    say("attention, reference test case")
+    gold = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "layers_test_n64_h12_cta160.json")))
+    heads, n = 12, 64
+    i = torch.arange(heads * n * 64 * 64, dtype=torch.float64)
+    ramp = (6.0 / 4095.0 * (i % 4096) - 2.0).view(heads, n * 64, 64).permute(1, 0, 2)      # token-major [T, H, d]
+    k = v = ramp.to(torch.float16)
+    qs = (ramp * lh.LOG2E).to(torch.float16)                    # the kernel's softmax is base 2
+    sb = capi.seq_prefix_blocks([4096])
+    idx = np.asarray(gold["to_select_index"], dtype=np.int32)
+    pos = np.asarray(gold["to_select_index_position"], dtype=np.int32)
+    fi = np.asarray(gold["from_select_index"], dtype=np.int32)
+    fp = np.asarray(gold["from_select_index_position"], dtype=np.int32)
+    dev = lambda a: torch.from_numpy(a).cuda()
+    qp, kp = lh.pack_heads(qs.cuda(), sb), lh.pack_heads(k.cuda(), sb)
+    vp = lh.pack_heads(v.cuda(), sb, transpose_v=True)
+    ref = oa.csr_attention(qs, k, v, sb.tolist(), idx, pos, 1, scale=1.0 / lh.LOG2E)
+    outs = []
+    for plan in ((dev(fi), dev(fp)), (None, None)):             # the reference's partition / the kernel's own schedule
+        out = torch.full((4096, heads * 64), float("nan"), dtype=torch.float16, device="cuda")
+        capi.bs_attention_fwd(qp, kp, vp, out, dev(sb), heads, dev(idx), dev(pos), 1, plan[0], plan[1], None)
+        torch.cuda.synchronize()
+        outs.append(out.float().cpu())
+        assert (outs[-1] - ref).abs().max().item() <= 2e-2
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_attention_large_logits_and_constant_v(capi):
     """Online softmax must survive scores of several hundred; constant V must come back exactly."""
     say("attention extremes")
