@@ -122,6 +122,8 @@ std::map<std::string, std::pair<double, int64_t>> timing_collect() {
       auto& slot = out[r.key];
       slot.first += double(ms) * 1000.0;
       slot.second += 1;
+    } else {
+      (void)hipGetLastError();          // a pair that measured nothing must not surface as the next call's error
     }
     (void)hipEventDestroy(r.a);
     (void)hipEventDestroy(r.b);
@@ -165,6 +167,7 @@ ScopedGpuTimer::~ScopedGpuTimer() {
     (void)hipEventSynchronize(b);
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, a, b) == hipSuccess) *slot_ += ms * 1000.0f;
+    else (void)hipGetLastError();
   }
   if (deferred_) {
     Deferred& d = deferred();

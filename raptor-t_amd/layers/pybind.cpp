@@ -56,7 +56,10 @@ PYBIND11_MODULE(raptor_t, m) {
           const bool ok = hipEventSynchronize(eb) == hipSuccess && hipEventElapsedTime(&ms, ea, eb) == hipSuccess;
           (void)hipEventDestroy(ea);
           (void)hipEventDestroy(eb);
-          if (!ok) throw std::runtime_error("the events were never given to a launch, or the launch failed");
+          if (!ok) {
+            (void)hipGetLastError();      // the failed query must not surface in the caller's next GPU call
+            throw std::runtime_error("the events were never given to a launch, or the launch failed");
+          }
           return double(ms) * 1000.0;
         },
         "Waits for the stop event, returns the microseconds between the two and destroys both.");
