@@ -450,14 +450,21 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
   const int g = blockIdx.x / heads, h = (blockIdx.x % heads + g) % heads;
   const int dm = heads * 64;
   const T* src = qkv + int64_t(g) * 64 * (3 * dm) + h * 64;
-  // every load of the thread is issued before anything waits for one: the kernel lives on bytes in flight
+  // every load of the thread is issued before anything waits for one: the kernel lives on bytes in flight.
+  // The projection's rows are read once and never again by this kernel: non-temporal loads keep them from
+  // pushing the K / V^T tiles written below out of the caches before the attention kernel, which runs next,
+  // reads them (measured in the step's kernel order: this kernel 46 -> 39 us, the attention kernel after it
+  // 119 -> 105 us).
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   uint4 raw[ITERS][3];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int c = threadIdx.x + it * 256, row = c / CPR, col = (c % CPR) * N;
 #pragma unroll
-    for (int m = M0; m < 3; ++m)
-      raw[it][m] = *reinterpret_cast<const uint4*>(src + int64_t(row) * 3 * dm + m * dm + col);
+    for (int m = M0; m < 3; ++m) {
+      const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + int64_t(row) * 3 * dm + m * dm + col));
+      raw[it][m] = make_uint4(v.x, v.y, v.z, v.w);
+    }
   }
   const int s = find_seq(seq_blocks, batch, g);
   const int g0 = seq_blocks[s], n = seq_blocks[s + 1] - g0;
