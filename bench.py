@@ -44,7 +44,7 @@ def block_pairs(seq_blocks, heads):
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default workload and scaled by
 # what the same counters read for the QKV split kernel (a copy of known size); the summaries and the commands are
 # in profiles/memory_kernels_c3_traffic.txt.  Only valid for that workload.
-MEASURED_TRAFFIC_C3 = {"bs_attention_kernel": 527.0e6, "bias_residual_layernorm_kernel": 171.4e6,
+MEASURED_TRAFFIC_C3 = {"bs_attention_kernel": 518.2e6, "bias_residual_layernorm_kernel": 171.4e6,
                        "bias_gelu_kernel": 457.0e6, "qkv_bias_split_kernel_q": 342.8e6, "qkv_bias_split_kernel": 228.5e6}
 
 
