@@ -398,13 +398,15 @@ template <typename T>
 __device__ inline QPlan q_plan(const Args<T>& a, const Unit& u, int lane) {
   QPlan q;
   if (a.q_rows) {
-    // raw projection rows: fragment (nt, c), lane l = dims 16c + 8(l >> 5) .. +7 of query 32nt + (l & 31),
-    // a 16-byte run of the token's row
+    // raw projection rows: request k = 4 nt + c takes the 128-byte head slices of queries 8k .. 8k + 7 whole,
+    // eight lanes per query (eight cache lines per request; taking MFMA fragments straight from the rows
+    // would touch 32 lines per request and return four times as slowly).  finish_q turns the eight
+    // requests' registers into fragments through LDS.
     const int ld = a.heads * 384;                                   // bytes per token row of [T, 3 * heads * 64]
-    q.voff = (lane & 31) * ld + (lane >> 5) * 16;
+    q.voff = (lane >> 3) * ld + (lane & 7) * 16;
     q.soff = (u.g0 + u.i) * 64 * ld + u.h * 128;
     q.nt_step = 32 * ld;
-    q.c_step = 32;
+    q.c_step = 8 * ld;
   } else {
     q.voff = lane * 16;
     q.soff = (u.g0 * a.heads + u.h * u.n + u.i) * 8192;
@@ -425,12 +427,28 @@ __device__ inline void request_q(const Args<T>& a, const Buffers<T>& b, const Un
   for (int k = 0; k < 8; ++k) qf[k >> 2][k & 3] = fetch_q<T>(b, q, k);
 }
 
-// (x + bias) * scale in fp32, rounded once: the arithmetic of the split kernel.  qbias = LDS copy of the bias.
+// What the queries-from-rows route keeps in LDS: a copy of the query bias and, per wave, room for one 64 x 64
+// query tile in row order (rows Q_STAGE_PITCH bytes apart).
+constexpr int Q_STAGE_PITCH = 144;
+constexpr int Q_STAGE_BYTES = 64 * Q_STAGE_PITCH;
+template <typename T> struct QSide { const T* bias; char* stage; };
+
+// Rows -> fragments through the wave's own LDS room (no other wave touches it: LDS operations of one wave
+// execute in order), then (x + bias) * scale in fp32, rounded once: the arithmetic of the split kernel.
 template <typename T>
-__device__ inline void finish_q(const Args<T>& a, const T* qbias, const Unit& u, int lane,
+__device__ inline void finish_q(const Args<T>& a, const QSide<T>& qs, const Unit& u, int lane,
                                 typename Mma<T>::v8 (&qf)[2][4]) {
   typedef typename Mma<T>::v8 v8;
   if (!a.q_rows) return;
+  const T* qbias = qs.bias;
+  {
+    char* wr = qs.stage + (lane >> 3) * Q_STAGE_PITCH + (lane & 7) * 16;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) *reinterpret_cast<v8*>(wr + k * 8 * Q_STAGE_PITCH) = qf[k >> 2][k & 3];
+    const char* rd = qs.stage + (lane & 31) * Q_STAGE_PITCH + (lane >> 5) * 16;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) qf[k >> 2][k & 3] = *reinterpret_cast<const v8*>(rd + (k >> 2) * 32 * Q_STAGE_PITCH + (k & 3) * 32);
+  }
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const v8 bb = *reinterpret_cast<const v8*>(qbias + u.h * 64 + c * 16 + (lane >> 5) * 8);
@@ -674,7 +692,7 @@ __device__ inline bool sums_finite(const State& st) { return !__any(!(st.l[0] < 
 
 // moving-maximum loop on entries first, first + step, ... of row r
 template <typename T, bool MASKED>
-__device__ inline void slow_row(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Row& r, int first, int step,
+__device__ inline void slow_row(const Args<T>& a, const Buffers<T>& b, const QSide<T>& qbias, const Row& r, int first, int step,
                                 int lane, bool have_q, typename Mma<T>::v8 (&qf)[2][4], State& st) {
   if (!have_q) {
     request_q<T>(a, b, r.u, lane, qf);
@@ -689,7 +707,7 @@ __device__ inline void slow_row(const Args<T>& a, const Buffers<T>& b, const T* 
 // from or to another row.  False: the row has to be run with the moving-maximum loop instead (more
 // than 64 entries for this wave, or scores that outgrew the reference); the state is then undefined.
 template <typename T>
-__device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Row& r, int first, int step,
+__device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const QSide<T>& qbias, const Row& r, int first, int step,
                                 int lane, State& st) {
   Tiles<T> t;
   state_init(st);
@@ -728,7 +746,7 @@ __device__ inline Row describe(const Args<T>& a, const Unit& u) {
 // One wave, one unit, all of its key blocks.  FAST: pipelined loop; false = the unit has to be run
 // again with FAST = false (nothing was written).
 template <typename T, bool MASKED, bool FAST>
-__device__ inline bool run_solo(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Unit& u, int lane) {
+__device__ inline bool run_solo(const Args<T>& a, const Buffers<T>& b, const QSide<T>& qbias, const Unit& u, int lane) {
   const Row r = describe<T>(a, u);
   State st;
   if (FAST) {
@@ -744,7 +762,7 @@ __device__ inline bool run_solo(const Args<T>& a, const Buffers<T>& b, const T* 
 // Four waves, one unit: wave w streams key blocks w, w+4, ...; tree merge through LDS.  FAST:
 // pipelined loop; false (the same in all four waves) = the unit has to be run again with FAST = false.
 template <typename T, bool MASKED, bool FAST>
-__device__ inline bool run_split4(const Args<T>& a, const Buffers<T>& b, const T* qbias, const Unit& u, int lane,
+__device__ inline bool run_split4(const Args<T>& a, const Buffers<T>& b, const QSide<T>& qbias, const Unit& u, int lane,
                                   int wave, float* park) {
   const Row r = describe<T>(a, u);
   State st;
@@ -801,6 +819,7 @@ __device__ inline bool run_split4(const Args<T>& a, const Buffers<T>& b, const T
     const int64_t stride = int64_t(a.heads) * 64;
     store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w);
   }
+  __syncthreads();                                    // the park is read: the next item may stage its queries there
   return true;
 }
 
@@ -819,21 +838,24 @@ __device__ inline int request_ticket_if(__amdgpu_buffer_rsrc_t counter, int lane
 // Persistent workgroups (two per CU).
 template <typename T, bool MASKED>
 __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
-  // 34816 bytes: two parked wave states for the global-row merge
-  __shared__ __attribute__((aligned(16))) float park[2 * 68 * 64];
+  // 36864 bytes with two uses that never overlap in time: two parked wave states (2 x 17408 bytes) of the merge
+  // that ends a row shared by the four waves, and each wave's room for a query tile in row order (finish_q)
+  static_assert(4 * Q_STAGE_BYTES >= 2 * 68 * 64 * int(sizeof(float)), "the park must hold two wave states");
+  __shared__ __attribute__((aligned(16))) float park[4 * Q_STAGE_BYTES / 4];
   __shared__ Geometry geo;
-  __shared__ __attribute__((aligned(16))) T qbias[MAX_HEADS_QROWS * 64];
+  __shared__ __attribute__((aligned(16))) T qbias_lds[MAX_HEADS_QROWS * 64];
   __shared__ int s_item;
   __shared__ int redo[4][REDO_SLOTS];                 // per wave: units put aside for the moving-maximum loop
   __shared__ int redo_rows[REDO_SLOTS];               // per workgroup: global rows put aside
   __shared__ uint8_t s_redo[REDO_ENTRIES];            // LPT plan: entries of the workgroup's slice to run again
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const QSide<T> qbias{qbias_lds, reinterpret_cast<char*>(park) + wave * Q_STAGE_BYTES};
 
   // geometry: prefix blocks, the list of rows that are not global rows, the sequences that have global rows
   int* const row_base = reinterpret_cast<int*>(park);            // per sequence: rows listed before it (scratch use of the park)
   for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
   if (a.q_rows)
-    for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias[i] = a.q_bias[i];
+    for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias_lds[i] = a.q_bias[i];
   __syncthreads();
   for (int i = threadIdx.x; i < a.batch; i += 256) {
     int t = 64;
