@@ -298,7 +298,13 @@ int rt_pooler_dense_tanh(const void* pooled, const void* weight_t, const void* b
  * rt_pipeline_acquire blocks the host until that layer's CSR is queued, then makes the
  * caller's stream wait on the event.  device < 0 keeps everything on the host (the
  * returned pointers are host pointers) so the ordering logic can be exercised without
- * a GPU.  async = 0 builds the CSR inside rt_pipeline_acquire instead. */
+ * a GPU.  async = 0 builds the CSR inside rt_pipeline_acquire instead.
+ * rt_pipeline_release(layer, stream) is called after the kernel that reads the layer's CSR has been launched
+ * on `stream`.  Each layer keeps two CSR buffers; the one a batch used is written again two batches later,
+ * once every reader of that batch has finished: the pipeline records one event per batch, behind the release
+ * of layer n_layers - 1, or, for a batch that never got that far, at the next rt_pipeline_publish behind the
+ * batch's last release.  The layers of one batch are therefore launched on one stream, in any order that ends
+ * with the last layer, and all before the next publish. */
 typedef struct rt_pipeline rt_pipeline;
 int rt_pipeline_create(rt_pipeline** p, int n_layers, int heads, int plan_mode, int max_pos,
                        int policy, int async, int device);

@@ -34,8 +34,7 @@ struct Slot {                 // one generation of one layer's CSR
   int* dev_pos = nullptr;
   int64_t cap_idx = 0, cap_pos = 0;
   hipEvent_t copied = nullptr;     // recorded on the copy stream after the H2D copies
-  hipEvent_t consumed = nullptr;   // recorded by rt_pipeline_release on the compute stream
-  bool consumed_pending = false;
+  bool consumed_pending = false;   // a kernel that reads the slot has been launched (rt_pipeline_release)
 };
 
 struct Layer {
@@ -63,6 +62,15 @@ struct rt_pipeline {
   std::mutex geo_m;
   std::vector<int> seq_blocks;
   int64_t gen = 0;
+  // "Every kernel of generation g that reads a slot has finished": one event per slot parity, recorded on the
+  // compute stream once per generation, behind the last layer's kernel (rt_pipeline_release of layer
+  // n_layers - 1), or, for a generation whose last layer never ran, by the next rt_pipeline_publish behind
+  // whatever that generation did launch.  One record per batch instead of one per layer: a record costs the
+  // stream about 6 us.  Guarded by geo_m.
+  hipEvent_t step_consumed[2] = {nullptr, nullptr};
+  int64_t step_recorded_gen[2] = {-1, -1};
+  int64_t last_release_gen = -1;
+  void* last_release_stream = nullptr;
   std::vector<Layer> layers;
   explicit rt_pipeline(int n) : sem_count(n, 0), layers(n) {}
 };
@@ -94,10 +102,9 @@ int free_slot(rt_pipeline* p, Slot& s) {
 
 int ensure_capacity(rt_pipeline* p, Slot& s, int64_t need_idx, int64_t need_pos) {
   if (need_idx <= s.cap_idx && need_pos <= s.cap_pos) return RT_OK;
-  hipEvent_t copied = s.copied, consumed = s.consumed;
+  hipEvent_t copied = s.copied;
   free_slot(p, s);
   s.copied = copied;
-  s.consumed = consumed;
   const int64_t ci = need_idx + need_idx / 2 + 64, cp = need_pos + need_pos / 2 + 64;
   if (p->device >= 0) {
     HIP_TRY(hipHostMalloc((void**)&s.host_idx, ci * sizeof(int), hipHostMallocDefault));
@@ -128,8 +135,8 @@ int build_layer(rt_pipeline* p, int l, int64_t gen, const std::vector<int>& sb) 
     wait_consumer = s.consumed_pending;
     s.consumed_pending = false;
   }
-  if (p->device >= 0 && wait_consumer)             // the kernel that read this slot two batches ago
-    HIP_TRY(hipEventSynchronize(s.consumed));
+  if (p->device >= 0 && wait_consumer)             // the kernels that read this slot two batches ago
+    HIP_TRY(hipEventSynchronize(p->step_consumed[gen & 1]));
   if (p->device >= 0 && s.copied) HIP_TRY(hipEventSynchronize(s.copied));
   rc = ensure_capacity(p, s, need_idx, need_pos);
   if (rc) return rc;
@@ -194,11 +201,15 @@ int rt_pipeline_create(rt_pipeline** out, int n_layers, int heads, int plan_mode
   if (device >= 0) {
     hipError_t e = hipSetDevice(device);
     if (e != hipSuccess) { delete p; return rt::fail(RT_EIO, "hipSetDevice(%d): %s", device, hipGetErrorString(e)); }
+    for (hipEvent_t& ev : p->step_consumed)
+      if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+        rt_pipeline_destroy(p);
+        return rt::fail(RT_EIO, "could not create the pipeline's events");
+      }
     for (Layer& L : p->layers) {
       bool ok = hipStreamCreateWithFlags(&L.copy_stream, hipStreamNonBlocking) == hipSuccess;
       for (Slot& s : L.slot) {
         ok = ok && hipEventCreateWithFlags(&s.copied, hipEventDisableTiming) == hipSuccess;
-        ok = ok && hipEventCreateWithFlags(&s.consumed, hipEventDisableTiming) == hipSuccess;
       }
       if (!ok) { rt_pipeline_destroy(p); return rt::fail(RT_EIO, "could not create the copy stream / events"); }
     }
@@ -216,6 +227,12 @@ int rt_pipeline_publish(rt_pipeline* p, const int* seq_blocks, int batch) {
   if (rc) return rc;
   {
     std::lock_guard<std::mutex> lk(p->geo_m);
+    // the generation that ends here launched readers but never reached its last layer: close it now
+    const int64_t g = p->gen;
+    if (p->device >= 0 && p->last_release_gen == g && p->step_recorded_gen[g & 1] != g) {
+      HIP_TRY(hipEventRecord(p->step_consumed[g & 1], (hipStream_t)p->last_release_stream));
+      p->step_recorded_gen[g & 1] = g;
+    }
     p->seq_blocks.assign(seq_blocks, seq_blocks + batch + 1);
     p->gen += 1;
   }
@@ -282,12 +299,16 @@ int rt_pipeline_release(rt_pipeline* p, int layer, void* stream) {
   {
     std::lock_guard<std::mutex> lk(p->geo_m);
     gen = p->gen;
+    p->last_release_gen = gen;
+    p->last_release_stream = stream;
+    if (layer == p->n_layers - 1) {
+      HIP_TRY(hipEventRecord(p->step_consumed[gen & 1], (hipStream_t)stream));
+      p->step_recorded_gen[gen & 1] = gen;
+    }
   }
   Layer& L = p->layers[layer];
   std::lock_guard<std::mutex> lk(L.m);
-  Slot& s = L.slot[gen & 1];
-  HIP_TRY(hipEventRecord(s.consumed, (hipStream_t)stream));
-  s.consumed_pending = true;
+  L.slot[gen & 1].consumed_pending = true;
   return RT_OK;
 }
 
@@ -304,16 +325,22 @@ int rt_pipeline_destroy(rt_pipeline* p) {
   }
   if (p->device >= 0) {
     (void)hipSetDevice(p->device);
+    // readers of the slots may still run: close the open generation and wait for both
+    if (p->last_release_gen >= 0 && p->step_recorded_gen[p->last_release_gen & 1] != p->last_release_gen &&
+        p->step_consumed[p->last_release_gen & 1])
+      (void)hipEventRecord(p->step_consumed[p->last_release_gen & 1], (hipStream_t)p->last_release_stream);
+    for (hipEvent_t ev : p->step_consumed)
+      if (ev) (void)hipEventSynchronize(ev);
     for (Layer& L : p->layers) {
       if (L.copy_stream) (void)hipStreamSynchronize(L.copy_stream);
       for (Slot& s : L.slot) {
-        if (s.consumed_pending) (void)hipEventSynchronize(s.consumed);
         free_slot(p, s);
         if (s.copied) (void)hipEventDestroy(s.copied);
-        if (s.consumed) (void)hipEventDestroy(s.consumed);
       }
       if (L.copy_stream) (void)hipStreamDestroy(L.copy_stream);
     }
+    for (hipEvent_t ev : p->step_consumed)
+      if (ev) (void)hipEventDestroy(ev);
   } else {
     for (Layer& L : p->layers)
       for (Slot& s : L.slot) free_slot(p, s);
