@@ -190,20 +190,37 @@ def cpu_baseline_membound(steps=20):
             "host_cpu_count": os.cpu_count(), "cpu_model": cpu_model()}
 
 
+DTYPES = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+
+# The encoder workloads by name: (hidden, heads, ffn, layers, dtype, lengths(util), positions the plans are drawn for)
+ENCODER_WORKLOADS = {
+    "c3": (768, 12, 3072, 12, "f16", lambda ut: ut.uniform_lengths(16, 512, 4096, seed=0), 4096),
+    "c5": (1024, 16, 4096, 24, "bf16", lambda ut: ut.uniform_lengths(4, 2048, 16384, seed=0), 16384),
+}
+
+
+def encoder_inputs(mb, hidden, ffn, layers, dt, seq_lens):
+    """The synthetic inputs of an encoder workload: per layer N(0, 0.02) weights in `dt` on the GPU, then the packed
+    N(0, 1) hidden states, all from one generator seeded with 0 (the parity tests of the headline workloads build
+    their inputs through this function, so what they check is what is timed)."""
+    g = torch.Generator().manual_seed(0)
+    layers_w = [mb.random_layer_weights(hidden, ffn, g, dtype=dt) for _ in range(layers)]
+    x0 = torch.randn(sum(seq_lens), hidden, generator=g).to(dt).cuda()
+    return layers_w, x0
+
+
 def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos=4096):
     pkg = graft.load_package()
     mb = importlib.import_module("raptor_t_amd.modeling_bert")
     ut = importlib.import_module("raptor_t_amd.util")
-    dt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[dtype]
-    g = torch.Generator().manual_seed(0)
-    layers_w = [mb.random_layer_weights(hidden, ffn, g, dtype=dt) for _ in range(layers)]
+    dt = DTYPES[dtype]
+    layers_w, x0 = encoder_inputs(mb, hidden, ffn, layers, dt, seq_lens)
     mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, max_pos)
     enc = mb.BertEncoder.from_weights(layers_w, heads, async_=not args.sync_index, eps=1e-5)
     meta = mb.cxx.MetaData()
     t = sum(seq_lens)
     block_limit = args.block_limit
     spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, block_limit, heads)
-    x0 = torch.randn(t, hidden, generator=g).to(dt).cuda()
     hidden_states = torch.empty_like(x0)
     new = lambda w: torch.empty(t, w, dtype=dt, device="cuda")
     inter, tmp, attn = new(ffn), new(hidden), new(hidden)
@@ -715,14 +732,16 @@ def main():
         sys.exit(2)
     ut = importlib.import_module("raptor_t_amd.util") if graft.load_package() else None
     if args.workload == "c3":
-        res = run_encoder(args, "c3: 12-layer BigBird-base, batch 16, len U[512,4096]", 768, 12, 3072, 12, "f16",
-                          ut.uniform_lengths(16, 512, 4096, seed=0))
+        hidden, heads, ffn, layers, dtype, lens, max_pos = ENCODER_WORKLOADS["c3"]
+        res = run_encoder(args, "c3: 12-layer BigBird-base, batch 16, len U[512,4096]", hidden, heads, ffn, layers, dtype,
+                          lens(ut), max_pos=max_pos)
     elif args.workload == "c1":
         res = run_encoder(args, "c1: one BigBird-base layer, batch 1 x 1024 tokens, fp32 (the accuracy mode)", 768, 12,
                           3072, 1, "f32", [1024])
     elif args.workload == "c5":
-        res = run_encoder(args, "c5: 24-layer BigBird-large shape, batch 4, len U[2048,16384], bf16", 1024, 16, 4096,
-                          24, "bf16", ut.uniform_lengths(4, 2048, 16384, seed=0), max_pos=16384)
+        hidden, heads, ffn, layers, dtype, lens, max_pos = ENCODER_WORKLOADS["c5"]
+        res = run_encoder(args, "c5: 24-layer BigBird-large shape, batch 4, len U[2048,16384], bf16", hidden, heads, ffn,
+                          layers, dtype, lens(ut), max_pos=max_pos)
     elif args.workload == "ref_e2e":
         import random
         lens = ut.generate_array_with_avg(3584, 16, 4096, random.Random(0))

@@ -125,6 +125,14 @@ int rt_meta_partition_lpt(const int* seq_blocks, int batch, int heads, int n_wg,
  * a caller that builds plans of its own calls this first. */
 int rt_meta_check_partition(const int* from_pos, const int* from_idx, int n_wg, int total_blocks, int heads);
 
+/* Host-side check of a to-block index before it is handed to an attention launch (no counterpart in the
+ * reference, whose kernels trust layers/multi_headed_attention.cpp:15-140): to_pos[plan_heads*NB+1] starts at 0,
+ * never decreases, leaves no row empty and ends inside to_idx[idx_len]; every entry of the row of (plan head,
+ * sequence s, block i) names a block of sequence s, 0 .. n_s-1.  RT_EINVAL otherwise.  The attention kernels clamp
+ * a block id they are handed, so a bad entry reads the wrong tile rather than fault; row bounds they take as given. */
+int rt_meta_check_to_index(const int* to_idx, const int* to_pos, int64_t idx_len, const int* seq_blocks, int batch,
+                           int plan_heads);
+
 /* --------------------------------------------------------------------- GPU kernels */
 
 /* Replaces kernels::add_bias_and_transpose_kernel (layers/kernels/
@@ -156,8 +164,10 @@ int rt_unpack_head_tiles(const void* packed, void* dst, const int* seq_blocks_de
  * every tensor fp32, fp32 matrix instructions; an accuracy mode, about ten times slower.
  * Limits of one launch (RT_EINVAL beyond them): batch <= 1024 sequences, total_blocks <= 4096
  * (262144 tokens), total_blocks * heads * 24576 < 2^31 (byte offsets are 32-bit).  The first launch
- * on a device without from_idx/from_pos allocates 256 KiB of counters that the library keeps
- * (rt_bs_attention_fwd_no_alloc does not). */
+ * on a device without from_idx/from_pos allocates 384 KiB of counters that the library keeps
+ * (rt_bs_attention_fwd_no_alloc does not): a ring of 64 sets, one per launch, each left zeroed by the
+ * launch that used it.  Launches may overlap on any number of streams and threads, in any order, as
+ * long as no more than 64 of them are in flight on one device at a time. */
 int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out,
                         const int* seq_blocks_dev, int batch, int total_blocks, int heads,
                         const int* to_idx, const int* to_pos, int plan_heads,
@@ -301,10 +311,12 @@ int rt_pooler_dense_tanh(const void* pooled, const void* weight_t, const void* b
  * a GPU.  async = 0 builds the CSR inside rt_pipeline_acquire instead.
  * rt_pipeline_release(layer, stream) is called after the kernel that reads the layer's CSR has been launched
  * on `stream`.  Each layer keeps two CSR buffers; the one a batch used is written again two batches later,
- * once every reader of that batch has finished: the pipeline records one event per batch, behind the release
- * of layer n_layers - 1, or, for a batch that never got that far, at the next rt_pipeline_publish behind the
- * batch's last release.  The layers of one batch are therefore launched on one stream, in any order that ends
- * with the last layer, and all before the next publish. */
+ * once every reader of that batch has finished: per batch the pipeline records one event on every stream
+ * layers were released on, behind the release of layer n_layers - 1, and for whatever was released after
+ * that (or in a batch that never got that far) at the next rt_pipeline_publish.  The layers of one batch may
+ * be launched in any order, on any streams, more than once, all before the next publish.
+ * rt_pipeline_set_index_check(p, 1): every CSR a worker builds goes through rt_meta_check_to_index before it
+ * is uploaded, and a failure comes back from rt_pipeline_acquire (a debugging aid; off by default). */
 typedef struct rt_pipeline rt_pipeline;
 int rt_pipeline_create(rt_pipeline** p, int n_layers, int heads, int plan_mode, int max_pos,
                        int policy, int async, int device);
@@ -312,6 +324,7 @@ int rt_pipeline_publish(rt_pipeline* p, const int* seq_blocks, int batch);
 int rt_pipeline_acquire(rt_pipeline* p, int layer, void* stream, const int** to_idx,
                         const int** to_pos, int* plan_heads, double* host_wait_us);
 int rt_pipeline_release(rt_pipeline* p, int layer, void* stream);
+int rt_pipeline_set_index_check(rt_pipeline* p, int on);
 int rt_pipeline_destroy(rt_pipeline* p);
 
 #ifdef __cplusplus

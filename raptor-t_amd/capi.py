@@ -22,12 +22,12 @@ RT_GEMM_TUNE_ALL = -1
 EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_time_next_launch", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
     "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
-    "rt_meta_partition_lpt", "rt_meta_check_partition", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
+    "rt_meta_partition_lpt", "rt_meta_check_partition", "rt_meta_check_to_index", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows", "rt_bs_attention_fwd_no_alloc",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm_set_retuning", "rt_gemm",
     "rt_gemm_bias_act", "rt_gemm_bt", "rt_sequence_pool", "rt_pooler_dense_tanh",
     "rt_pipeline_create", "rt_pipeline_publish", "rt_pipeline_acquire", "rt_pipeline_release",
-    "rt_pipeline_destroy",
+    "rt_pipeline_destroy", "rt_pipeline_set_index_check",
 ]
 
 
@@ -59,6 +59,7 @@ def lib():
         L.rt_meta_block_costs.argtypes = [i32p, I, i32p, i64p]
         L.rt_meta_partition_lpt.argtypes = [i32p, I, I, I, i32p, i32p]
         L.rt_meta_check_partition.argtypes = [i32p, i32p, I, I, I]
+        L.rt_meta_check_to_index.argtypes = [i32p, i32p, L64, i32p, I, I]
         L.rt_qkv_bias_split.argtypes = [vp, vp, vp, vp, vp, vp, I, I, I, F, I, vp]
         L.rt_unpack_head_tiles.argtypes = [vp, vp, vp, I, I, I, I, I, vp]
         L.rt_bs_attention_fwd.argtypes = [vp, vp, vp, vp, vp, I, I, I, vp, vp, I, vp, vp, I, I, vp]
@@ -83,6 +84,7 @@ def lib():
                                           ctypes.POINTER(ctypes.c_double)]
         L.rt_pipeline_release.argtypes = [vp, I, vp]
         L.rt_pipeline_destroy.argtypes = [vp]
+        L.rt_pipeline_set_index_check.argtypes = [vp, I]
         _lib = L
     return _lib
 
@@ -163,6 +165,15 @@ def check_partition(from_pos, from_idx, total_blocks, heads):
     if len(ids) != total_blocks * heads or len(pos) < 2:
         raise ValueError("from_idx needs total_blocks * heads entries and from_pos at least two")
     check(lib().rt_meta_check_partition(_p(pos), _p(ids), len(pos) - 1, total_blocks, heads))
+
+
+def check_to_index(to_idx, to_pos, seq_blocks, plan_heads):
+    """Raises RaptorError unless (to_idx, to_pos) is a to-block index of the batch `seq_blocks`: one non-empty row
+    per (plan head, block), every entry a block of the row's own sequence."""
+    idx, pos, sb = _i32(to_idx), _i32(to_pos), _i32(seq_blocks)
+    if len(sb) < 2 or len(pos) != plan_heads * int(sb[-1]) + 1:
+        raise ValueError("to_pos needs plan_heads * total_blocks + 1 entries")
+    check(lib().rt_meta_check_to_index(_p(idx), _p(pos), len(idx), _p(sb), len(sb) - 1, plan_heads))
 
 
 # ------------------------------------------------------------------------------- GPU kernels
@@ -433,6 +444,9 @@ class Pipeline:
     def release(self, layer, stream=None):
         st = ctypes.c_void_p(0) if self.device < 0 else (stream if stream is not None else _stream())
         check(lib().rt_pipeline_release(self._h, layer, st))
+
+    def set_index_check(self, on):
+        check(lib().rt_pipeline_set_index_check(self._h, 1 if on else 0))
 
     def close(self):
         if self._h:

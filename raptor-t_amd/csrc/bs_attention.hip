@@ -344,17 +344,20 @@ template <typename T> struct Args {
   // optional: Q taken from the QKV projection's own output rows [tokens, 3 * heads * 64] (columns
   // 0 .. heads*64-1), bias added and scale applied while loading; q is then unused
   const T* q_rows; const T* q_bias; float q_scale;
-  int* queues;                           // QUEUE_INTS ints of device memory, all zero when the kernel starts
-  int* queues_clear;                     // the counters of a later launch: this launch puts them back to zero
+  int* queues;                           // QUEUE_INTS ints of device memory, all zero when the kernel starts and when it ends
 };
 
 constexpr int MAX_BATCH = 1024;         // sequences per launch (geometry is kept in LDS)
 constexpr int MAX_BLOCKS = 4096;        // 64-token blocks per launch (the row table is kept in LDS)
 constexpr int MAX_HEADS_QROWS = 64;     // heads whose query bias fits the LDS copy
-// Queue counters of one launch: 16 of them (tickets of the 8 global-row queues, then of the 8 unit
-// queues), each alone in a 256-byte line: tickets of one line are served one after the other.
+// Queue counters of one launch: 24 of them (tickets of the 8 global-row queues, tickets of the 8 unit
+// queues, then per XCD the number of its workgroups that have finished), each alone in a 256-byte line:
+// tickets of one line are served one after the other.  Every counter is only ever touched by the
+// workgroups of one XCD, through atomics that its L2 executes; the last workgroup of an XCD to finish
+// puts that XCD's three counters back to zero, so a launch leaves its counters as it found them.
 constexpr int QUEUE_STRIDE = 64;                    // ints between two counters
-constexpr int QUEUE_INTS = 16 * QUEUE_STRIDE;
+constexpr int QUEUE_COUNTERS = 24;
+constexpr int QUEUE_INTS = QUEUE_COUNTERS * QUEUE_STRIDE;
 constexpr int REDO_SLOTS = 32;          // units a wave may put aside for the moving-maximum loop before it runs them
 constexpr int REDO_ENTRIES = 2048;      // LPT plan: entries per workgroup whose pipelined attempt is tracked
 
@@ -968,7 +971,6 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
   const int xcd = blockIdx.x & 7;
   const __amdgpu_buffer_rsrc_t gq = ticket_counter(a.queues + xcd * QUEUE_STRIDE);          // this XCD's global-row queue
   const __amdgpu_buffer_rsrc_t uq = ticket_counter(a.queues + (8 + xcd) * QUEUE_STRIDE);    // this XCD's unit queue
-  if (blockIdx.x == 0 && threadIdx.x < 16) a.queues_clear[threadIdx.x * QUEUE_STRIDE] = 0;
 
   // phase 1: global rows, one per workgroup.  A pair = the first and the last row of one (sequence,
   // head): both stream the same K / V^T tiles, so they are consecutive tickets of the same XCD.
@@ -1144,6 +1146,22 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       n_redo = 0;
     }
   }
+
+  // This workgroup draws no more tickets.  The last workgroup of the XCD to get here puts the XCD's counters
+  // back to zero for the next launch that is handed them (same L2, same kind of access as the tickets).
+  __syncthreads();
+  if (wave == 0) {
+    const __amdgpu_buffer_rsrc_t done = ticket_counter(a.queues + (16 + xcd) * QUEUE_STRIDE);
+    const int finished = __builtin_amdgcn_readfirstlane(request_ticket(done, lane));
+    if (finished == int(gridDim.x >> 3) - 1) {
+      // nobody else touches them any more: read each (an addition of nothing) and take that much away
+      const int g = __builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(0, gq, lane * 4, 0, 1);
+      const int u = __builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(0, uq, lane * 4, 0, 1);
+      (void)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(-g, gq, lane * 4, 0, 0);
+      (void)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(-u, uq, lane * 4, 0, 0);
+      (void)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(-(finished + 1), done, lane * 4, 0, 0);
+    }
+  }
 }
 
 // Two persistent workgroups per CU, a multiple of 8 so that every XCD gets the same number.
@@ -1159,10 +1177,11 @@ unsigned plan_free_workgroups() {
 }
 
 // Queue counters of the library's own launches: a ring of slots, so that launches which overlap on
-// different streams do not share counters.  A launch leaves its slot used; launch i clears the slot
-// that launch i + QUEUE_SLOTS / 2 will take.
+// different streams do not share counters.  A launch leaves its slot zeroed (the kernel's last
+// workgroups do that), so the slots need no order among the launches that use them; what the ring cannot
+// cover is more than QUEUE_SLOTS attention launches of the library in flight on one device at the same time.
 constexpr int QUEUE_SLOTS = 64;
-int* library_queues(int* err, int** clear) {
+int* library_queues(int* err) {
   static int* base[64] = {};
   static unsigned next[64] = {};
   static std::mutex mu;
@@ -1177,7 +1196,6 @@ int* library_queues(int* err, int** clear) {
     base[dev] = p;
   }
   const unsigned slot = next[dev]++ % QUEUE_SLOTS;
-  *clear = base[dev] + ((slot + QUEUE_SLOTS / 2) % QUEUE_SLOTS) * QUEUE_INTS;
   return base[dev] + slot * QUEUE_INTS;
 }
 
@@ -1188,8 +1206,7 @@ namespace {
 int launch_attention(const void* q, const void* q_rows, const void* q_bias, float q_scale, const void* k, const void* vt,
                      void* out, const int* seq_blocks_dev, const int* seq_tokens_dev, int batch, int total_blocks,
                      int heads, const int* to_idx, const int* to_pos, int plan_heads, const int* from_idx,
-                     const int* from_pos, int n_wg, int dtype, void* stream, int* own_queues = nullptr,
-                     int* own_queues_clear = nullptr) {
+                     const int* from_pos, int n_wg, int dtype, void* stream, int* own_queues = nullptr) {
   RT_REQUIRE((q || (q_rows && q_bias)) && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1, RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d",
              batch, total_blocks, heads);
@@ -1213,7 +1230,6 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
   }
   unsigned grid;
   int* queues = nullptr;
-  int* queues_clear = nullptr;
   if (from_idx) {
     RT_REQUIRE(n_wg >= 1, RT_EINVAL, "balanced launch needs n_wg >= 1, got %d", n_wg);
     grid = unsigned(n_wg);
@@ -1221,10 +1237,9 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
     grid = plan_free_workgroups();
     if (own_queues) {
       queues = own_queues;
-      queues_clear = own_queues_clear;
     } else {
       int err = 0;
-      queues = library_queues(&err, &queues_clear);
+      queues = library_queues(&err);
       if (!queues) return rt::fail(RT_ENOMEM, "no device memory for the work queues (step %d)", err);
     }
   }
@@ -1232,13 +1247,13 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
   if (dtype == RT_F16) {
     Args<_Float16> a{(const _Float16*)q, (const _Float16*)k, (const _Float16*)vt, (_Float16*)out, seq_blocks_dev, batch,
                      heads, total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
-                     (const _Float16*)q_rows, (const _Float16*)q_bias, q_scale, queues, queues_clear};
+                     (const _Float16*)q_rows, (const _Float16*)q_bias, q_scale, queues};
     if (seq_tokens_dev) RT_LAUNCH((bs_attention_kernel<_Float16, true>), dim3(grid), dim3(256), 0, st, a);
     else RT_LAUNCH((bs_attention_kernel<_Float16, false>), dim3(grid), dim3(256), 0, st, a);
   } else {
     Args<__bf16> a{(const __bf16*)q, (const __bf16*)k, (const __bf16*)vt, (__bf16*)out, seq_blocks_dev, batch, heads,
                    total_blocks, to_idx, to_pos, plan_heads, from_idx, from_pos, seq_tokens_dev,
-                   (const __bf16*)q_rows, (const __bf16*)q_bias, q_scale, queues, queues_clear};
+                   (const __bf16*)q_rows, (const __bf16*)q_bias, q_scale, queues};
     if (seq_tokens_dev) RT_LAUNCH((bs_attention_kernel<__bf16, true>), dim3(grid), dim3(256), 0, st, a);
     else RT_LAUNCH((bs_attention_kernel<__bf16, false>), dim3(grid), dim3(256), 0, st, a);
   }
@@ -1278,12 +1293,11 @@ extern "C" int rt_bs_attention_fwd(const void* q, const void* k, const void* vt,
 }
 
 // ---- the entry point that allocates nothing -------------------------------------------------------
-// Its queue counters live in this array instead of the library's allocated ring.  First half: the
-// counters of the running launch, zeroed by a fill kernel ahead of every launch; second half: where
-// that launch's own clearing store goes (nobody reads it).  In host code the array's name is only a
-// stand-in: its address on a device comes from hipGetSymbolAddress, once per device.
-constexpr int NO_ALLOC_SCRATCH_INTS = 2 * QUEUE_INTS;
-static_assert(NO_ALLOC_SCRATCH_INTS * sizeof(int) == RT_NO_ALLOC_SCRATCH_BYTES, "header and kernel disagree on the scratch size");
+// Its queue counters live in this array instead of the library's allocated ring, zeroed by a fill kernel
+// ahead of every launch (whatever an earlier launch that was cut short may have left there).  In host code
+// the array's name is only a stand-in: its address on a device comes from hipGetSymbolAddress, once per device.
+constexpr int NO_ALLOC_SCRATCH_INTS = RT_NO_ALLOC_SCRATCH_BYTES / int(sizeof(int));
+static_assert(NO_ALLOC_SCRATCH_INTS >= QUEUE_INTS, "the scratch array must hold one launch's counters");
 static_assert(RT_NO_ALLOC_MAX_BATCH <= MAX_BATCH && RT_NO_ALLOC_MAX_BLOCKS <= MAX_BLOCKS, "header limits exceed the kernel's");
 static __device__ __align__(256) int scratch[NO_ALLOC_SCRATCH_INTS];
 
@@ -1317,9 +1331,9 @@ extern "C" int rt_bs_attention_fwd_no_alloc(const void* q, const void* k, const 
              RT_NO_ALLOC_MAX_BATCH, RT_NO_ALLOC_MAX_BLOCKS, RT_NO_ALLOC_MAX_BLOCKS * 64, batch, total_blocks);
   int* counters = no_alloc_scratch();
   if (!counters) return rt::fail(RT_EIO, "the address of the static scratch array is not available on this device");
-  hipLaunchKernelGGL(clear_queue_counters, dim3(1), dim3(QUEUE_INTS / QUEUE_STRIDE), 0, static_cast<hipStream_t>(stream), counters);
+  hipLaunchKernelGGL(clear_queue_counters, dim3(1), dim3(QUEUE_COUNTERS), 0, static_cast<hipStream_t>(stream), counters);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return rt::fail(RT_EIO, "clearing the queue counters failed: %s", hipGetErrorString(e));
   return launch_attention(q, nullptr, nullptr, 1.0f, k, vt, out, seq_blocks_dev, seq_tokens_dev, batch, total_blocks, heads,
-                          to_idx, to_pos, plan_heads, nullptr, nullptr, 0, dtype, stream, counters, counters + QUEUE_INTS);
+                          to_idx, to_pos, plan_heads, nullptr, nullptr, 0, dtype, stream, counters);
 }

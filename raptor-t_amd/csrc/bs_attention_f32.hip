@@ -88,7 +88,8 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
   const int g0 = a.seq_blocks[lo], n = a.seq_blocks[lo + 1] - g0;
   const int rem = unit - g0 * a.heads;
   const int h = rem / n, i = rem - h * n;
-  const int tail = MASKED ? a.seq_tokens[lo] - 64 * (n - 1) : 64;      // real tokens of the last block
+  // real tokens of the last block; at least one (a tile with every key masked has no finite maximum)
+  const int tail = MASKED ? min(max(a.seq_tokens[lo] - 64 * (n - 1), 1), 64) : 64;
   const int row = (a.plan_heads > 1 ? h : 0) * a.nb_total + g0 + i;
   const int p0 = a.to_pos[row], p1 = a.to_pos[row + 1];
   const int64_t head_base = (int64_t(g0) * a.heads + int64_t(h) * n) * 4096;
@@ -120,7 +121,7 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
   float m = -INFINITY, l = 0.f;
 
   for (int p = p0; p < p1; ++p) {
-    const int blk = a.to_idx[p];
+    const int blk = min(max(a.to_idx[p], 0), n - 1);   // a malformed index must not lead outside the (sequence, head)
     __syncthreads();                                   // the previous tile's readers are done
     stage_tile<false>(a.k + head_base + int64_t(blk) * 4096, ks);
     stage_tile<true>(a.vt + head_base + int64_t(blk) * 4096, vs);

@@ -422,4 +422,33 @@ int rt_meta_check_partition(const int* from_pos, const int* from_idx, int n_wg, 
   return RT_OK;
 }
 
+int rt_meta_check_to_index(const int* to_idx, const int* to_pos, int64_t idx_len, const int* seq_blocks, int batch,
+                           int plan_heads) {
+  RT_REQUIRE(to_idx && to_pos && seq_blocks, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(batch >= 1 && plan_heads >= 1 && idx_len >= 0, RT_EINVAL, "bad batch=%d / plan_heads=%d / idx_len=%lld", batch,
+             plan_heads, (long long)idx_len);
+  RT_REQUIRE(seq_blocks[0] == 0, RT_EINVAL, "block index: seq_blocks must start at 0, got %d", seq_blocks[0]);
+  for (int s = 0; s < batch; ++s)
+    RT_REQUIRE(seq_blocks[s + 1] > seq_blocks[s], RT_EINVAL, "block index: sequence %d has no blocks", s);
+  const int nb = seq_blocks[batch];
+  const int64_t rows = int64_t(plan_heads) * nb;
+  RT_REQUIRE(to_pos[0] == 0, RT_EINVAL, "block index: to_pos must start at 0, got %d", to_pos[0]);
+  RT_REQUIRE(to_pos[rows] <= idx_len, RT_EINVAL, "block index: to_pos ends at %d, to_idx holds %lld entries", to_pos[rows],
+             (long long)idx_len);
+  for (int hp = 0; hp < plan_heads; ++hp)
+    for (int s = 0; s < batch; ++s) {
+      const int n = seq_blocks[s + 1] - seq_blocks[s];
+      for (int i = 0; i < n; ++i) {
+        const int64_t row = int64_t(hp) * nb + seq_blocks[s] + i;
+        const int p0 = to_pos[row], p1 = to_pos[row + 1];
+        RT_REQUIRE(p1 > p0, RT_EINVAL, "block index: row %lld (plan head %d, sequence %d, block %d) is empty or to_pos decreases",
+                   (long long)row, hp, s, i);
+        for (int p = p0; p < p1; ++p)
+          RT_REQUIRE(to_idx[p] >= 0 && to_idx[p] < n, RT_EINVAL,
+                     "block index: entry %d of row %lld names block %d, the sequence has %d", p - p0, (long long)row, to_idx[p], n);
+      }
+    }
+  return RT_OK;
+}
+
 }  // extern "C"

@@ -62,15 +62,15 @@ struct rt_pipeline {
   std::mutex geo_m;
   std::vector<int> seq_blocks;
   int64_t gen = 0;
-  // "Every kernel of generation g that reads a slot has finished": one event per slot parity, recorded on the
-  // compute stream once per generation, behind the last layer's kernel (rt_pipeline_release of layer
-  // n_layers - 1), or, for a generation whose last layer never ran, by the next rt_pipeline_publish behind
-  // whatever that generation did launch.  One record per batch instead of one per layer: a record costs the
-  // stream about 6 us.  Guarded by geo_m.
-  hipEvent_t step_consumed[2] = {nullptr, nullptr};
-  int64_t step_recorded_gen[2] = {-1, -1};
-  int64_t last_release_gen = -1;
-  void* last_release_stream = nullptr;
+  // "Every kernel of generation g that reads a slot has finished": per slot parity one event for every stream
+  // readers were launched on.  A release marks its stream's entry open; the open entries of the current
+  // generation are recorded (each on its own stream) behind the last layer's kernel (rt_pipeline_release of
+  // layer n_layers - 1), and whatever was released after that, or in a generation whose last layer never ran,
+  // by the next rt_pipeline_publish.  One record per batch and stream instead of one per layer: a record costs
+  // the stream about 6 us.  Guarded by geo_m.
+  struct Closing { void* stream; hipEvent_t ev; bool open; };
+  std::vector<Closing> closing[2];
+  std::atomic<bool> check_index{false};     // rt_pipeline_set_index_check
   std::vector<Layer> layers;
   explicit rt_pipeline(int n) : sem_count(n, 0), layers(n) {}
 };
@@ -78,6 +78,17 @@ struct rt_pipeline {
 namespace {
 
 int plan_heads_of(const rt_pipeline* p) { return p->plan_mode == RT_PLAN_REFERENCE ? 1 : p->heads; }
+
+// Records the open entries of one slot parity, each behind everything queued on its stream.  Caller holds geo_m.
+int close_readers_locked(rt_pipeline* p, int parity) {
+  for (rt_pipeline::Closing& c : p->closing[parity]) {
+    if (!c.open) continue;
+    hipError_t e = hipEventRecord(c.ev, (hipStream_t)c.stream);
+    if (e != hipSuccess) return rt::fail(RT_EIO, "hipEventRecord (readers finished): %s", hipGetErrorString(e));
+    c.open = false;
+  }
+  return RT_OK;
+}
 
 #define HIP_TRY(expr)                                                              \
   do {                                                                             \
@@ -135,14 +146,24 @@ int build_layer(rt_pipeline* p, int l, int64_t gen, const std::vector<int>& sb) 
     wait_consumer = s.consumed_pending;
     s.consumed_pending = false;
   }
-  if (p->device >= 0 && wait_consumer)             // the kernels that read this slot two batches ago
-    HIP_TRY(hipEventSynchronize(p->step_consumed[gen & 1]));
+  if (p->device >= 0 && wait_consumer) {           // the kernels that read this slot two batches ago
+    std::vector<hipEvent_t> readers;
+    {
+      std::lock_guard<std::mutex> lk(p->geo_m);
+      for (const rt_pipeline::Closing& c : p->closing[gen & 1]) readers.push_back(c.ev);
+    }
+    for (hipEvent_t ev : readers) HIP_TRY(hipEventSynchronize(ev));
+  }
   if (p->device >= 0 && s.copied) HIP_TRY(hipEventSynchronize(s.copied));
   rc = ensure_capacity(p, s, need_idx, need_pos);
   if (rc) return rc;
   rc = rt_meta_build_to_index(sb.data(), batch, ph, p->plan_mode, uint32_t(l), p->max_pos, p->policy, nullptr,
                               s.host_idx, s.cap_idx, s.host_pos, s.cap_pos);
   if (rc) return rc;
+  if (p->check_index) {
+    rc = rt_meta_check_to_index(s.host_idx, s.host_pos, need_idx, sb.data(), batch, ph);
+    if (rc) return rc;
+  }
   if (p->device >= 0) {
     HIP_TRY(hipMemcpyAsync(s.dev_idx, s.host_idx, need_idx * sizeof(int), hipMemcpyHostToDevice, L.copy_stream));
     HIP_TRY(hipMemcpyAsync(s.dev_pos, s.host_pos, need_pos * sizeof(int), hipMemcpyHostToDevice, L.copy_stream));
@@ -201,11 +222,6 @@ int rt_pipeline_create(rt_pipeline** out, int n_layers, int heads, int plan_mode
   if (device >= 0) {
     hipError_t e = hipSetDevice(device);
     if (e != hipSuccess) { delete p; return rt::fail(RT_EIO, "hipSetDevice(%d): %s", device, hipGetErrorString(e)); }
-    for (hipEvent_t& ev : p->step_consumed)
-      if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
-        rt_pipeline_destroy(p);
-        return rt::fail(RT_EIO, "could not create the pipeline's events");
-      }
     for (Layer& L : p->layers) {
       bool ok = hipStreamCreateWithFlags(&L.copy_stream, hipStreamNonBlocking) == hipSuccess;
       for (Slot& s : L.slot) {
@@ -227,11 +243,11 @@ int rt_pipeline_publish(rt_pipeline* p, const int* seq_blocks, int batch) {
   if (rc) return rc;
   {
     std::lock_guard<std::mutex> lk(p->geo_m);
-    // the generation that ends here launched readers but never reached its last layer: close it now
-    const int64_t g = p->gen;
-    if (p->device >= 0 && p->last_release_gen == g && p->step_recorded_gen[g & 1] != g) {
-      HIP_TRY(hipEventRecord(p->step_consumed[g & 1], (hipStream_t)p->last_release_stream));
-      p->step_recorded_gen[g & 1] = g;
+    // readers of the generation that ends here which no record covers yet (its last layer never ran, or layers
+    // were launched again after it): close them now
+    if (p->device >= 0) {
+      rc = close_readers_locked(p, int(p->gen & 1));
+      if (rc) return rc;
     }
     p->seq_blocks.assign(seq_blocks, seq_blocks + batch + 1);
     p->gen += 1;
@@ -299,16 +315,29 @@ int rt_pipeline_release(rt_pipeline* p, int layer, void* stream) {
   {
     std::lock_guard<std::mutex> lk(p->geo_m);
     gen = p->gen;
-    p->last_release_gen = gen;
-    p->last_release_stream = stream;
+    std::vector<rt_pipeline::Closing>& cl = p->closing[gen & 1];
+    size_t k = 0;
+    while (k < cl.size() && cl[k].stream != stream) ++k;
+    if (k == cl.size()) {
+      hipEvent_t ev = nullptr;
+      HIP_TRY(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+      cl.push_back(rt_pipeline::Closing{stream, ev, false});
+    }
+    cl[k].open = true;
     if (layer == p->n_layers - 1) {
-      HIP_TRY(hipEventRecord(p->step_consumed[gen & 1], (hipStream_t)stream));
-      p->step_recorded_gen[gen & 1] = gen;
+      int rc = close_readers_locked(p, int(gen & 1));
+      if (rc) return rc;
     }
   }
   Layer& L = p->layers[layer];
   std::lock_guard<std::mutex> lk(L.m);
   L.slot[gen & 1].consumed_pending = true;
+  return RT_OK;
+}
+
+int rt_pipeline_set_index_check(rt_pipeline* p, int on) {
+  RT_REQUIRE(p, RT_EINVAL, "NULL pipeline");
+  p->check_index = on != 0;
   return RT_OK;
 }
 
@@ -325,12 +354,11 @@ int rt_pipeline_destroy(rt_pipeline* p) {
   }
   if (p->device >= 0) {
     (void)hipSetDevice(p->device);
-    // readers of the slots may still run: close the open generation and wait for both
-    if (p->last_release_gen >= 0 && p->step_recorded_gen[p->last_release_gen & 1] != p->last_release_gen &&
-        p->step_consumed[p->last_release_gen & 1])
-      (void)hipEventRecord(p->step_consumed[p->last_release_gen & 1], (hipStream_t)p->last_release_stream);
-    for (hipEvent_t ev : p->step_consumed)
-      if (ev) (void)hipEventSynchronize(ev);
+    // readers of the slots may still run: close what is open and wait for every stream's readers
+    for (int parity = 0; parity < 2; ++parity) {
+      (void)close_readers_locked(p, parity);
+      for (const rt_pipeline::Closing& c : p->closing[parity]) (void)hipEventSynchronize(c.ev);
+    }
     for (Layer& L : p->layers) {
       if (L.copy_stream) (void)hipStreamSynchronize(L.copy_stream);
       for (Slot& s : L.slot) {
@@ -339,8 +367,8 @@ int rt_pipeline_destroy(rt_pipeline* p) {
       }
       if (L.copy_stream) (void)hipStreamDestroy(L.copy_stream);
     }
-    for (hipEvent_t ev : p->step_consumed)
-      if (ev) (void)hipEventDestroy(ev);
+    for (int parity = 0; parity < 2; ++parity)
+      for (const rt_pipeline::Closing& c : p->closing[parity]) (void)hipEventDestroy(c.ev);
   } else {
     for (Layer& L : p->layers)
       for (Slot& s : L.slot) free_slot(p, s);

@@ -64,26 +64,48 @@ static void require_index(const torch::Tensor& t, const char* name, int64_t nume
                                 std::to_string(numel));
 }
 
-// The host's work plan, checked once per tensor pair (same storage, same version, same size as the pair
-// checked last: nothing to do).  Costs one device-to-host copy the first time a plan is seen.
+// The host's work plan, checked once per tensor pair.  "The pair checked last" is recognised by its storages
+// (held through weak references: while one is held, the allocator cannot hand the same storage object to a new
+// tensor, and a storage that has died is never taken for a live one), offsets, sizes and versions.  Costs one
+// device-to-host copy the first time a plan is seen.
 static void require_valid_partition(const torch::Tensor& from_idx, const torch::Tensor& from_pos, int n_wg, int block_num,
                                     int head_num) {
-  struct Key { const void* idx; const void* pos; int64_t n_idx, n_pos; uint32_t v_idx, v_pos; };
+  typedef c10::weak_intrusive_ptr<c10::StorageImpl> WeakStorage;
+  struct Key {
+    WeakStorage idx, pos;
+    int64_t off_idx = 0, off_pos = 0, n_idx = 0, n_pos = 0;
+    uint32_t v_idx = 0, v_pos = 0;
+    int n_wg = 0, block_num = 0, head_num = 0;
+    Key() : idx(WeakStorage(c10::intrusive_ptr<c10::StorageImpl>())), pos(WeakStorage(c10::intrusive_ptr<c10::StorageImpl>())) {}
+  };
   static std::mutex m;
-  static Key last = {nullptr, nullptr, 0, 0, 0, 0};
-  const Key now = {from_idx.data_ptr(), from_pos.data_ptr(), from_idx.numel(), from_pos.numel(),
-                   uint32_t(from_idx._version()), uint32_t(from_pos._version())};
+  static Key last;
+  const c10::StorageImpl* si = from_idx.storage().unsafeGetStorageImpl();
+  const c10::StorageImpl* sp = from_pos.storage().unsafeGetStorageImpl();
   {
     std::lock_guard<std::mutex> lk(m);
-    if (now.idx == last.idx && now.pos == last.pos && now.n_idx == last.n_idx && now.n_pos == last.n_pos &&
-        now.v_idx == last.v_idx && now.v_pos == last.v_pos)
+    if (!last.idx.expired() && !last.pos.expired() && last.idx._unsafe_get_target() == si &&
+        last.pos._unsafe_get_target() == sp && last.off_idx == from_idx.storage_offset() &&
+        last.off_pos == from_pos.storage_offset() && last.n_idx == from_idx.numel() && last.n_pos == from_pos.numel() &&
+        last.v_idx == uint32_t(from_idx._version()) && last.v_pos == uint32_t(from_pos._version()) && last.n_wg == n_wg &&
+        last.block_num == block_num && last.head_num == head_num)
       return;
   }
   const torch::Tensor idx_h = from_idx.cpu(), pos_h = from_pos.cpu();
   check(rt_meta_check_partition(pos_h.data_ptr<int>(), idx_h.data_ptr<int>(), n_wg, block_num, head_num),
         "balanced attention: bad work plan");
   std::lock_guard<std::mutex> lk(m);
-  last = now;
+  last.idx = from_idx.storage().getWeakStorageImpl();
+  last.pos = from_pos.storage().getWeakStorageImpl();
+  last.off_idx = from_idx.storage_offset();
+  last.off_pos = from_pos.storage_offset();
+  last.n_idx = from_idx.numel();
+  last.n_pos = from_pos.numel();
+  last.v_idx = uint32_t(from_idx._version());
+  last.v_pos = uint32_t(from_pos._version());
+  last.n_wg = n_wg;
+  last.block_num = block_num;
+  last.head_num = head_num;
 }
 
 namespace {

@@ -37,12 +37,16 @@ MultiHeadedAttention::MultiHeadedAttention(torch::Tensor, torch::Tensor, torch::
 std::pair<std::vector<int>, std::vector<int>> MultiHeadedAttention::GenerateSparseBlockIndex() const {
   const std::vector<int> sb = TensorSet::get_instance()->seq_len_info_;
   if (sb.size() < 2) throw std::runtime_error("GenerateSparseBlockIndex: no batch has been published");
-  const int batch = int(sb.size()) - 1, heads = int(num_attention_heads_);
+  // the plan the index pipeline of this lane draws (MetaData.set_plan): this function returns what the workers build
+  int plan_mode = RT_PLAN_HF, policy = RT_POLICY_REFERENCE_PATCHED, max_pos = 4096;
+  Semaphore::get_instance()->get_plan(&plan_mode, &policy, &max_pos);
+  const int batch = int(sb.size()) - 1;
+  const int plan_heads = plan_mode == RT_PLAN_REFERENCE ? 1 : int(num_attention_heads_);
   int64_t n_idx = 0, n_pos = 0;
-  kernels::check(rt_meta_to_index_size(sb.data(), batch, heads, &n_idx, &n_pos), "rt_meta_to_index_size");
+  kernels::check(rt_meta_to_index_size(sb.data(), batch, plan_heads, &n_idx, &n_pos), "rt_meta_to_index_size");
   std::vector<int> idx(n_idx), pos(n_pos);
-  kernels::check(rt_meta_build_to_index(sb.data(), batch, heads, RT_PLAN_HF, uint32_t(layer_idx_), 4096,
-                                        RT_POLICY_REFERENCE_PATCHED, nullptr, idx.data(), n_idx, pos.data(), n_pos),
+  kernels::check(rt_meta_build_to_index(sb.data(), batch, plan_heads, plan_mode, uint32_t(layer_idx_), max_pos, policy,
+                                        nullptr, idx.data(), n_idx, pos.data(), n_pos),
                  "rt_meta_build_to_index");
   return {idx, pos};
 }

@@ -172,5 +172,13 @@ PYBIND11_MODULE(raptor_t, m) {
                       layers::Semaphore::get_instance(lane)->set_plan(plan_mode, policy, max_pos);
                   },
                   py::arg("plan_mode") = int(RT_PLAN_HF), py::arg("policy") = int(RT_POLICY_REFERENCE_PATCHED),
-                  py::arg("max_pos") = 4096);
+                  py::arg("max_pos") = 4096)
+      .def_static("set_index_check",
+                  [](bool on) {
+                    for (int lane = 0; lane < layers::LANES; ++lane)
+                      layers::Semaphore::get_instance(lane)->set_index_check(on);
+                  },
+                  py::arg("on"),
+                  "Debugging aid: every block index the workers build is checked on the host before it is uploaded; a "
+                  "malformed one makes the attention layer raise instead of launching.");
 }

@@ -43,6 +43,19 @@ void Semaphore::set_plan(int plan_mode, int policy, int max_pos) {
   if (pipeline_) { rt_pipeline_destroy(pipeline_); pipeline_ = nullptr; }
 }
 
+void Semaphore::get_plan(int* plan_mode, int* policy, int* max_pos) {
+  std::lock_guard<std::mutex> lk(mutex_);
+  *plan_mode = plan_mode_;
+  *policy = policy_;
+  *max_pos = max_pos_;
+}
+
+void Semaphore::set_index_check(bool on) {
+  std::lock_guard<std::mutex> lk(mutex_);
+  index_check_ = on;
+  if (pipeline_) check(rt_pipeline_set_index_check(pipeline_, on ? 1 : 0), "rt_pipeline_set_index_check");
+}
+
 void Semaphore::ensure_pipeline_locked() {
   if (layer_cond.empty()) throw std::runtime_error("Semaphore: no attention layer has registered");
   const int n_layers = layer_cond.rbegin()->first + 1;
@@ -53,6 +66,7 @@ void Semaphore::ensure_pipeline_locked() {
   if (hipGetDevice(&device) != hipSuccess) throw std::runtime_error("Semaphore: no HIP device");
   check(rt_pipeline_create(&pipeline_, n_layers, heads, plan_mode_, max_pos_, policy_, async_ ? 1 : 0, device),
         "rt_pipeline_create");
+  check(rt_pipeline_set_index_check(pipeline_, index_check_ ? 1 : 0), "rt_pipeline_set_index_check");
   pipeline_layers_ = n_layers;
   pipeline_heads_ = heads;
   pipeline_async_ = async_;

@@ -36,6 +36,10 @@ class Semaphore {
   void terminate();
   // plan mode / policy / max positions used for the next pipeline that is created
   void set_plan(int plan_mode, int policy, int max_pos);
+  void get_plan(int* plan_mode, int* policy, int* max_pos);
+  // debugging aid: every block index the workers build is checked on the host (rt_meta_check_to_index) before its
+  // upload; a malformed one makes Wait throw instead of reaching a kernel
+  void set_index_check(bool on);
   static Ptr get_instance();            // the current micro-batch lane's (tensor_set.h)
   static Ptr get_instance(int lane);
 
@@ -46,7 +50,7 @@ class Semaphore {
   std::map<int, int> layer_cond;      // registered layers -> heads
   rt_pipeline* pipeline_ = nullptr;
   int pipeline_layers_ = 0, pipeline_heads_ = 0;
-  bool pipeline_async_ = true, async_ = true;
+  bool pipeline_async_ = true, async_ = true, index_check_ = false;
   int plan_mode_ = RT_PLAN_HF, policy_ = RT_POLICY_REFERENCE_PATCHED, max_pos_ = 4096;
   std::vector<int> last_batch_;
   static Ptr instance_[2];

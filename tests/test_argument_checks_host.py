@@ -104,6 +104,40 @@ def test_partition_check_accepts_lpt_plans_and_names_what_is_wrong(capi):
         capi.check_partition(pos, ids[:-1], nb, heads)
 
 
+def test_to_index_check_accepts_built_indices_and_names_what_is_wrong(capi):
+    sb = capi.seq_prefix_blocks([832, 64, 1024, 320])
+    for plan_heads, mode in ((3, capi.RT_PLAN_HF), (1, capi.RT_PLAN_REFERENCE)):
+        idx, pos = capi.build_to_index(sb, plan_heads, mode=mode, seed=4)
+        capi.check_to_index(idx, pos, sb, plan_heads)
+        row = 2                                                 # block 2 of the 13-block sequence: a sparse row
+        bad = idx.copy()
+        bad[pos[row] + 1] = 13                                  # one past the sequence's last block
+        with pytest.raises(capi.RaptorError, match="names block 13"):
+            capi.check_to_index(bad, pos, sb, plan_heads)
+        bad = idx.copy()
+        bad[pos[13]] = 1                                        # the one-block sequence has only block 0
+        with pytest.raises(capi.RaptorError, match="names block 1"):
+            capi.check_to_index(bad, pos, sb, plan_heads)
+        bad = idx.copy()
+        bad[pos[row]] = -1
+        with pytest.raises(capi.RaptorError, match="names block -1"):
+            capi.check_to_index(bad, pos, sb, plan_heads)
+        p2 = pos.copy()
+        p2[row + 1] = p2[row]
+        with pytest.raises(capi.RaptorError, match="empty"):
+            capi.check_to_index(idx, p2, sb, plan_heads)
+        p2 = pos.copy()
+        p2[-1] += 5
+        with pytest.raises(capi.RaptorError, match="to_idx holds"):
+            capi.check_to_index(idx, p2, sb, plan_heads)
+        p2 = pos.copy()
+        p2[0] = 1
+        with pytest.raises(capi.RaptorError, match="start at 0"):
+            capi.check_to_index(idx, p2, sb, plan_heads)
+        with pytest.raises(ValueError):
+            capi.check_to_index(idx, pos[:-1], sb, plan_heads)
+
+
 def test_layer_launchers_refuse_bad_tensors(kernels):
     """The shims under the reference's kernel names (layers/kernels/kernel.h) check device, layout, dtype and sizes
     before they time or launch anything; on this machine every tensor is a host tensor, so each call must raise."""

@@ -147,6 +147,7 @@ def _host_csr(ptr, n):
 def test_pipeline_host_mode_builds_every_layer(capi, async_):
     heads, layers = 4, 6
     pipe = capi.Pipeline(layers, heads, async_=async_, device=-1)
+    pipe.set_index_check(True)                    # every CSR the pipeline builds passes rt_meta_check_to_index
     try:
         for lens in ([768, 1024], [4096], [64, 832, 2048, 128]):
             sb = capi.seq_prefix_blocks(lens)

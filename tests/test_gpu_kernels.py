@@ -669,6 +669,41 @@ def test_pipeline_on_device(capi):
     pipe.close()
 
 
+def test_pipeline_keeps_a_slot_until_late_readers_finish(capi):
+    """A layer launched AGAIN after the batch's last layer was released (a second, partial pass without a new
+    publish) is a reader no closing record covered when the per-batch event was tied to the last layer alone: two
+    publishes later the worker would overwrite the slot while that reader still waits on the GPU.  The reader here
+    is a device copy of the slot queued behind a sleeping kernel; it must see the batch it acquired."""
+    say("pipeline late reader")
+    import ctypes
+    from ctypes import c_void_p
+    hip = ctypes.CDLL("libamdhip64.so")
+    heads, layers = 2, 3
+    pipe = capi.Pipeline(layers, heads, device=0)
+    sb_a, sb_b, sb_c = (capi.seq_prefix_blocks(l) for l in ([832, 1024], [1280], [1024, 768]))
+    pipe.publish(sb_a)
+    for layer in range(layers):
+        pipe.acquire(layer)
+        pipe.release(layer)                                  # the last layer closes the batch
+    idx_p, pos_p, ph, _ = pipe.acquire(0)                    # second, partial pass: layer 0 only
+    n_idx, n_pos = capi.to_index_size(sb_a, ph)
+    seen = torch.zeros(n_idx, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda._sleep(int(2.0e8))                            # about 0.1 s: the reader is queued, not running
+    assert hip.hipMemcpyAsync(c_void_p(seen.data_ptr()), c_void_p(idx_p), n_idx * 4, 3, c_void_p(stream)) == 0
+    pipe.release(0)
+    pipe.publish(sb_b)
+    pipe.acquire(0)
+    pipe.release(0)
+    pipe.publish(sb_c)                                       # the workers now rebuild the slots batch A used
+    idx_c, _, _, _ = pipe.acquire(0)
+    assert idx_c == idx_p                                    # batch C sits in the buffer batch A used
+    torch.cuda.synchronize()
+    want_idx, _ = capi.build_to_index(sb_a, ph, seed=0)
+    assert np.array_equal(seen.cpu().numpy(), want_idx)
+    pipe.close()
+
+
 def test_attention_random_geometries(capi):
     """Twenty seeded draws of batch geometry (1 to 7 sequences of 1 to 40 blocks, so sparse and full-attention
     sequences mix), head count, dtype, plan mode, schedule (the kernel's own / a work plan of random size) and

@@ -120,6 +120,30 @@ def test_large_configuration_geometry_through_layer_api(pkg, mb, ut):
     lh.check_stack_output(out, want, dtype)
 
 
+def test_generate_sparse_block_index_follows_the_published_plan(pkg, mb, ut):
+    """BertAttention.generate_sparse_block_index (the reference's GenerateSparseBlockIndex,
+    layers/multi_headed_attention.cpp:15-140, as a callable) returns the index the workers build for the published
+    batch: plan mode, policy and position count of MetaData.set_plan, seed = layer index."""
+    say("generate_sparse_block_index")
+    hidden, heads, ffn, dtype = 256, 4, 512, torch.float16
+    g = torch.Generator().manual_seed(5)
+    w = {k: v.to(dtype).cuda() for k, v in ol.random_layer_weights(hidden, ffn, g).items()}
+    seq_lens = [8192, 832, 1024]                               # 8192 and 1024 take the plan drawn for max_pos positions
+    for max_pos in (16384, 8192):
+        mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, max_pos)
+        try:
+            layer = mb.BertLayer.from_weights(w, heads, 3, async_=True)
+            meta = mb.cxx.MetaData()
+            spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, 32, heads)
+            meta.update_meta_data(sum(seq_lens), spi[-1] + 1, total_comp, spi)
+            idx, pos = layer.attention.generate_sparse_block_index()
+            want_idx, want_pos = md.hf_to_index(seq_lens, 3, heads, max_pos=max_pos)
+            assert np.array_equal(np.asarray(idx), want_idx) and np.array_equal(np.asarray(pos), want_pos)
+            meta.terminate_thread()
+        finally:
+            mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, 4096)
+
+
 def test_two_stream_micro_batches_match_one_stream(mb, ut):
     """BertEncoder.call_two_streams (the batch cut in two micro-batches, each on a stream and a lane of per-batch
     state of its own) gives the bits of the ordinary call for every sequence, matches the oracle, works for a batch
@@ -551,3 +575,73 @@ def test_padded_batch_of_several_sequences_matches_huggingface_per_sequence(mb, 
         say("  sequence", s, "tokens", real, "err", err)
         assert err <= 2e-2
         assert bool((got[s, real:] == 0).all())
+
+
+def _run_headline_workload(pkg, mb, ut, name, two_streams):
+    """bench.py's encoder workload `name` once through the layer API (asynchronous block-index pipeline, the step
+    bench.py times); returns (hidden, heads, layers, dtype, lengths, positions, x0 fp32 on the host, the layers'
+    weights as fp32 on the host, output on the host as fp32)."""
+    import bench
+    hidden, heads, ffn, layers, dtype, lens, max_pos = bench.ENCODER_WORKLOADS[name]
+    dt, seq_lens = bench.DTYPES[dtype], lens(ut)
+    layers_w, x0 = bench.encoder_inputs(mb, hidden, ffn, layers, dt, seq_lens)
+    block_limit, eps = 1024, 1e-5                              # bench.py's defaults
+    mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, max_pos)
+    try:
+        enc = mb.BertEncoder.from_weights(layers_w, heads, async_=True, eps=eps)
+        meta = mb.cxx.MetaData()
+        t = sum(seq_lens)
+        new = lambda w: torch.empty(t, w, dtype=dt, device="cuda")
+        hs, tmp, inter, attn = x0.clone(), new(hidden), new(ffn), new(hidden)
+        if two_streams:
+            enc.call_two_streams(hs, seq_lens, block_limit, heads, tmp, inter, attn, test_info={}, balanced=False)
+        else:
+            spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, block_limit, heads)
+            meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+            enc(hs, t, block_limit, spi, spi_t, ppi_t, pp_t, tmp, inter, attn, test_info={}, balanced=False)
+        torch.cuda.synchronize()
+        meta.terminate_thread()
+    finally:
+        mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, 4096)
+    w32 = [{k: v.float().cpu() for k, v in w.items()} for w in layers_w]
+    return hidden, heads, layers, dt, seq_lens, max_pos, x0.float().cpu(), w32, hs.float().cpu()
+
+
+def _check_sampled_sequences(out, x0, w32, heads, seq_lens, picks, dt, max_pos):
+    """Sequences of a packed batch do not see each other: the oracle run on one sequence alone, through every layer,
+    is the expected value of that sequence's rows of the batch's output."""
+    starts = np.concatenate([[0], np.cumsum(seq_lens)])
+    for s in picks:
+        rows = slice(int(starts[s]), int(starts[s + 1]))
+        want = _oracle_encoder(x0[rows], w32, heads, [seq_lens[s]], 1e-5, dt, max_pos=max_pos)
+        err = (out[rows] - want).abs().max().item()
+        say("  sequence %d (%d tokens): max abs err %.3e" % (s, seq_lens[s], err))
+        lh.check_stack_output(out[rows], want, dt)
+
+
+def test_headline_workload_matches_oracle_on_sampled_sequences(pkg, mb, ut):
+    """The workload bench.py's default line times (12-layer BigBird-base, fp16, 16 sequences of 512 to 4096 tokens,
+    seed-0 weights, per-head plan seeded by the layer index, asynchronous pipeline), run once at full size; the
+    512-token sequence (every row lists every block) and the shortest sparse sequences are held to the per-element
+    bound against the oracle run on each of them alone through all 12 layers.  The reference's own end-to-end
+    benchmark (python/benchmark/end2end.py:80-92) compares no outputs."""
+    say("headline workload c3")
+    hidden, heads, layers, dt, seq_lens, max_pos, x0, w32, out = _run_headline_workload(pkg, mb, ut, "c3", False)
+    assert layers == 12 and len(seq_lens) == 16 and torch.isfinite(out).all()
+    order = sorted(range(len(seq_lens)), key=lambda s: seq_lens[s])
+    dense = [s for s in order if seq_lens[s] <= 704][:1]
+    sparse = [s for s in order if 768 <= seq_lens[s] <= 1500][:2]
+    assert dense and sparse, seq_lens
+    _check_sampled_sequences(out, x0, w32, heads, seq_lens, dense + sparse, dt, max_pos)
+
+
+@pytest.mark.parametrize("two_streams", [False, True])
+def test_large_workload_matches_oracle_on_its_shortest_sequence(pkg, mb, ut, two_streams):
+    """bench.py's `c5` workload (24-layer BigBird-large shape, bf16, 4 sequences of 2048 to 16384 tokens, plans drawn
+    for 16384 positions) at full size, on one stream and as two micro-batches on two streams; the shortest sequence
+    against the oracle run on it alone through all 24 layers (bound for a stack of bf16 layers)."""
+    say("large workload c5, two streams:", two_streams)
+    hidden, heads, layers, dt, seq_lens, max_pos, x0, w32, out = _run_headline_workload(pkg, mb, ut, "c5", two_streams)
+    assert layers == 24 and dt == torch.bfloat16 and torch.isfinite(out).all()
+    shortest = min(range(len(seq_lens)), key=lambda s: seq_lens[s])
+    _check_sampled_sequences(out, x0, w32, heads, seq_lens, [shortest], dt, max_pos)
