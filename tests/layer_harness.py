@@ -49,15 +49,17 @@ def outliers(got, want, dtype, k=1.0):
 
 
 def check_stack_output(got, want, dtype):
-    """Bound for the output of several layers.  fp16 and fp32: excess() with one ulp.  bf16, against an oracle that
+    """Bound for the output of a few layers.  fp16 and fp32: excess() with one ulp.  bf16, against an oracle that
     stores its tensors in bf16 too: at most 1 element in 10 000 outside max(2e-2, 2 ulp(|y|)), none further off than
-    two ulp of its row's largest value, rms error at most 4e-3 (measured: 3e-5, 2.0, 2.8e-3)."""
+    three ulp of its row's largest value, rms error at most 4e-3.  Measured on two layers: 3e-5, 2.0, 2.8e-3; the
+    largest error is a whole number of ulp, and which GEMM kernel the library picks on a box moves single roundings,
+    so the bound leaves one ulp above what was seen."""
     if dtype != torch.bfloat16:
         over = excess(got, want, dtype, k=1.0)
         assert over <= 0, over
         return
     share, worst, rms = outliers(got, want, dtype, k=2.0)
-    assert share <= 1e-4 and worst <= 2.0 and rms <= 4e-3, (share, worst, rms)
+    assert share <= 1e-4 and worst <= 3.0 and rms <= 4e-3, (share, worst, rms)
 
 
 def slot_tokens():

@@ -577,16 +577,19 @@ def test_padded_batch_of_several_sequences_matches_huggingface_per_sequence(mb, 
         assert bool((got[s, real:] == 0).all())
 
 
-def _run_headline_workload(pkg, mb, ut, name, two_streams):
+def _run_headline_workload(pkg, mb, ut, name, two_streams, keep_rows=None):
     """bench.py's encoder workload `name` once through the layer API (asynchronous block-index pipeline, the step
-    bench.py times); returns (hidden, heads, layers, dtype, lengths, positions, x0 fp32 on the host, the layers'
-    weights as fp32 on the host, output on the host as fp32)."""
+    bench.py times).  keep_rows (a slice of token rows, one stream only): the layers are called one by one, as
+    BertEncoder.__call__ calls them, and those rows of every layer's output are kept.  Returns (heads, layers,
+    dtype, lengths, positions, x0 fp32 on the host, the layers' weights as fp32 on the host, output on the host as
+    fp32, kept rows per layer)."""
     import bench
     hidden, heads, ffn, layers, dtype, lens, max_pos = bench.ENCODER_WORKLOADS[name]
     dt, seq_lens = bench.DTYPES[dtype], lens(ut)
     layers_w, x0 = bench.encoder_inputs(mb, hidden, ffn, layers, dt, seq_lens)
     block_limit, eps = 1024, 1e-5                              # bench.py's defaults
     mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, max_pos)
+    kept = []
     try:
         enc = mb.BertEncoder.from_weights(layers_w, heads, async_=True, eps=eps)
         meta = mb.cxx.MetaData()
@@ -598,50 +601,113 @@ def _run_headline_workload(pkg, mb, ut, name, two_streams):
         else:
             spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(seq_lens, 64, block_limit, heads)
             meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
-            enc(hs, t, block_limit, spi, spi_t, ppi_t, pp_t, tmp, inter, attn, test_info={}, balanced=False)
+            if keep_rows is None:
+                enc(hs, t, block_limit, spi, spi_t, ppi_t, pp_t, tmp, inter, attn, test_info={}, balanced=False)
+            else:
+                for l in enc.layer:
+                    l(hs, spi, spi_t, ppi_t, pp_t, inter, tmp, attn, block_limit, test_info={}, balanced=False)
+                    kept.append(hs[keep_rows].clone())
         torch.cuda.synchronize()
         meta.terminate_thread()
     finally:
         mb.cxx.MetaData.set_plan(pkg.capi.RT_PLAN_HF, pkg.capi.RT_POLICY_REFERENCE_PATCHED, 4096)
     w32 = [{k: v.float().cpu() for k, v in w.items()} for w in layers_w]
-    return hidden, heads, layers, dt, seq_lens, max_pos, x0.float().cpu(), w32, hs.float().cpu()
+    return heads, layers, dt, seq_lens, max_pos, x0.float().cpu(), w32, hs.float().cpu(), [k.float().cpu() for k in kept]
 
 
-def _check_sampled_sequences(out, x0, w32, heads, seq_lens, picks, dt, max_pos):
-    """Sequences of a packed batch do not see each other: the oracle run on one sequence alone, through every layer,
-    is the expected value of that sequence's rows of the batch's output."""
+def _rows_of(seq_lens, s):
     starts = np.concatenate([[0], np.cumsum(seq_lens)])
-    for s in picks:
-        rows = slice(int(starts[s]), int(starts[s + 1]))
-        want = _oracle_encoder(x0[rows], w32, heads, [seq_lens[s]], 1e-5, dt, max_pos=max_pos)
-        err = (out[rows] - want).abs().max().item()
-        say("  sequence %d (%d tokens): max abs err %.3e" % (s, seq_lens[s], err))
-        lh.check_stack_output(out[rows], want, dt)
+    return slice(int(starts[s]), int(starts[s + 1]))
 
 
 def test_headline_workload_matches_oracle_on_sampled_sequences(pkg, mb, ut):
     """The workload bench.py's default line times (12-layer BigBird-base, fp16, 16 sequences of 512 to 4096 tokens,
     seed-0 weights, per-head plan seeded by the layer index, asynchronous pipeline), run once at full size; the
     512-token sequence (every row lists every block) and the shortest sparse sequences are held to the per-element
-    bound against the oracle run on each of them alone through all 12 layers.  The reference's own end-to-end
-    benchmark (python/benchmark/end2end.py:80-92) compares no outputs."""
+    bound against the oracle run on each of them alone through all 12 layers (sequences of a packed batch do not
+    see each other).  The reference's own end-to-end benchmark (python/benchmark/end2end.py:80-92) compares no
+    outputs."""
     say("headline workload c3")
-    hidden, heads, layers, dt, seq_lens, max_pos, x0, w32, out = _run_headline_workload(pkg, mb, ut, "c3", False)
+    heads, layers, dt, seq_lens, max_pos, x0, w32, out, _ = _run_headline_workload(pkg, mb, ut, "c3", False)
     assert layers == 12 and len(seq_lens) == 16 and torch.isfinite(out).all()
     order = sorted(range(len(seq_lens)), key=lambda s: seq_lens[s])
     dense = [s for s in order if seq_lens[s] <= 704][:1]
     sparse = [s for s in order if 768 <= seq_lens[s] <= 1500][:2]
     assert dense and sparse, seq_lens
-    _check_sampled_sequences(out, x0, w32, heads, seq_lens, dense + sparse, dt, max_pos)
+    for s in dense + sparse:
+        rows = _rows_of(seq_lens, s)
+        want = _oracle_encoder(x0[rows], w32, heads, [seq_lens[s]], 1e-5, dt, max_pos=max_pos)
+        say("  sequence %d (%d tokens): max abs err %.3e" % (s, seq_lens[s], (out[rows] - want).abs().max().item()))
+        lh.check_stack_output(out[rows], want, dt)
 
 
-@pytest.mark.parametrize("two_streams", [False, True])
-def test_large_workload_matches_oracle_on_its_shortest_sequence(pkg, mb, ut, two_streams):
+def _large_workload_oracles(x_seq, w32, heads, length, max_pos):
+    """The shortest sequence of the large workload through all layers on the CPU, twice: every stored tensor rounded
+    to bf16 (what the layer objects store) and all in fp32 (the mathematical encoder)."""
+    stored = _oracle_encoder(x_seq, w32, heads, [length], 1e-5, torch.bfloat16, max_pos=max_pos)
+    sb = md.seq_prefix_blocks([length])
+    exact = x_seq.to(torch.bfloat16).float()
+    for li, w in enumerate(w32):
+        idx, pos = md.hf_to_index([length], li, heads, max_pos=max_pos)
+        exact = ol.encoder_layer(exact, w, heads, sb, idx, pos, heads, 1e-5)
+    return stored, exact
+
+
+def _check_deep_bf16_stack(got, stored, exact, what):
+    """24 layers in bf16: every stored tensor is rounded to 8 bits, a rounding that falls the other way is a
+    difference of 0.4 to 0.8 % of that element, and the differences add up from layer to layer like a random walk
+    (measured: rms 2.8e-3 after 2 layers, 1.1e-2 after 24), so no per-element bound holds against any oracle.  What
+    holds: the GPU path is as close to the all-fp32 encoder as the oracle that stores bf16 is (rms and largest
+    error within 1.5x of that oracle's own), and as close to that oracle as two such random walks are to each other
+    (rms within 2x of the oracle's distance to fp32)."""
+    rms = lambda a, b: (a - b).double().pow(2).mean().sqrt().item()
+    mx = lambda a, b: (a - b).abs().max().item()
+    floor_rms, floor_max = rms(stored, exact), mx(stored, exact)
+    say("  %s: rms to fp32 %.3e (bf16-storing oracle %.3e), max %.3e (%.3e), rms to the bf16-storing oracle %.3e"
+        % (what, rms(got, exact), floor_rms, mx(got, exact), floor_max, rms(got, stored)))
+    assert rms(got, exact) <= 1.5 * floor_rms and mx(got, exact) <= 1.5 * floor_max
+    assert rms(got, stored) <= 2.0 * floor_rms
+
+
+def test_large_workload_matches_oracle_layer_by_layer(pkg, mb, ut):
     """bench.py's `c5` workload (24-layer BigBird-large shape, bf16, 4 sequences of 2048 to 16384 tokens, plans drawn
-    for 16384 positions) at full size, on one stream and as two micro-batches on two streams; the shortest sequence
-    against the oracle run on it alone through all 24 layers (bound for a stack of bf16 layers)."""
-    say("large workload c5, two streams:", two_streams)
-    hidden, heads, layers, dt, seq_lens, max_pos, x0, w32, out = _run_headline_workload(pkg, mb, ut, "c5", two_streams)
-    assert layers == 24 and dt == torch.bfloat16 and torch.isfinite(out).all()
-    shortest = min(range(len(seq_lens)), key=lambda s: seq_lens[s])
-    _check_sampled_sequences(out, x0, w32, heads, seq_lens, [shortest], dt, max_pos)
+    for 16384 positions) at full size.  The shortest sequence is checked layer by layer: the oracle's layer l applied
+    to the GPU path's own input of layer l must give the GPU path's output of layer l, for each of the 24 layers with
+    its own plan.  A layer stores four bf16 tensors on the way; among the six million elements of one layer's output a
+    few sit behind a stored value that rounded the other way, so the bound per layer is: at most 1 element in 100 000
+    outside max(2e-2, two ulp), none further off than three ulp of its row's largest value, rms at most 4e-3.  The
+    final output is held to the bound for a deep bf16 stack."""
+    say("large workload c5, layer by layer")
+    import bench
+    seq_lens = bench.ENCODER_WORKLOADS["c5"][5](ut)
+    s = min(range(len(seq_lens)), key=lambda k: seq_lens[k])
+    rows = _rows_of(seq_lens, s)
+    heads, layers, dt, seq_lens, max_pos, x0, w32, out, kept = _run_headline_workload(pkg, mb, ut, "c5", False, rows)
+    assert layers == 24 and dt == torch.bfloat16 and len(kept) == 24 and torch.isfinite(out).all()
+    sb = md.seq_prefix_blocks([seq_lens[s]])
+    stats = []
+    for li in range(layers):
+        x_in = x0[rows].to(dt).float() if li == 0 else kept[li - 1]
+        idx, pos = md.hf_to_index([seq_lens[s]], li, heads, max_pos=max_pos)
+        want = ol.encoder_layer(x_in, w32[li], heads, sb, idx, pos, heads, 1e-5, store_dtype=dt)
+        stats.append(lh.outliers(kept[li], want, dt, k=2.0) + ((kept[li] - want).abs().max().item(),))
+    say("  per layer (share outside the per-element bound, worst in ulp of the row maximum, rms, max abs):")
+    for li, st in enumerate(stats):
+        say("   layer %2d: %.2e %.2f %.2e %.2e" % ((li,) + st))
+    for li, (share, worst, rms, _) in enumerate(stats):
+        assert share <= 1e-5 and worst <= 3.0 and rms <= 4e-3, (li, share, worst, rms)
+    assert torch.equal(kept[-1], out[rows])
+    stored, exact = _large_workload_oracles(x0[rows], w32, heads, seq_lens[s], max_pos)
+    _check_deep_bf16_stack(out[rows], stored, exact, "one stream")
+
+
+def test_large_workload_on_two_streams(pkg, mb, ut):
+    """The same workload through BertEncoder.call_two_streams (16 heads, bf16, rows of more than 64 blocks on two
+    micro-batch lanes): the shortest sequence against the oracles, bound for a deep bf16 stack."""
+    say("large workload c5, two streams")
+    heads, layers, dt, seq_lens, max_pos, x0, w32, out, _ = _run_headline_workload(pkg, mb, ut, "c5", True)
+    assert layers == 24 and torch.isfinite(out).all()
+    s = min(range(len(seq_lens)), key=lambda k: seq_lens[k])
+    rows = _rows_of(seq_lens, s)
+    stored, exact = _large_workload_oracles(x0[rows], w32, heads, seq_lens[s], max_pos)
+    _check_deep_bf16_stack(out[rows], stored, exact, "two streams")
