@@ -1,6 +1,6 @@
 """Benchmark of the block-sparse encoder hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2|c4|c5|ref_e2e|stream|overlap]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c1|c2|c4|c5|ref_e2e|stream|overlap|mfma_mix]
 
 Default workload `c3` is the headline configuration (benchmark config 3): the 12-layer BigBird-base fp16 encoder
 on a padding-free batch of 16 sequences with lengths uniform in [512, 4096] (multiples of
@@ -702,12 +702,63 @@ def run_overlap(args):
             "max_abs_diff_two_streams_vs_one": diff, "max_abs_diff_split_beside_projection": diff_split}
 
 
+def run_issue_floor(args):
+    """The figures behind the attention kernel's ceiling, from librt_probe.so (raptor-t_amd/csrc/probe_issue_floor.hip):
+    the time one SIMD needs per block pair for the pair's 32 matrix instructions alone, with the 64 exponentials,
+    with the 32 conversions, and with the packed row sums (the tile loop's whole instruction mix), every operand in
+    registers, on one and on two waves per SIMD, together with the clock the CUs held meanwhile.  Prints, asserts
+    nothing."""
+    import ctypes
+    path = os.path.join(ROOT, "raptor-t_amd", "lib", "librt_probe.so")
+    if not os.path.exists(path):
+        raise ImportError("%s is missing: run `make -C raptor-t_amd/csrc`" % path)
+    lib = ctypes.CDLL(path)
+    vp, I = ctypes.c_void_p, ctypes.c_int
+    lib.rt_probe_issue_floor.argtypes = [I, I, I, I, vp, vp, vp]
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.empty(cus * 512, dtype=torch.float32, device="cuda")
+    clocks = torch.zeros(2 * cus, dtype=torch.int64, device="cuda")
+    iters = 4000
+    st = torch.cuda.current_stream().cuda_stream
+    tick_hz = 100e6                                              # the constant-rate clock of wall_clock64()
+    names = ["32 mfma", "+ 64 v_exp_f32", "+ 32 v_cvt_pk_f16_f32", "+ 32 v_pk_add_f16 (the loop's mix)"]
+    rows = []
+    for wps in (1, 2):
+        for variant in range(4):
+            def launch(n=iters):
+                rc = lib.rt_probe_issue_floor(variant, wps, n, cus, out.data_ptr(), clocks.data_ptr(), st)
+                assert rc == 0, rc
+            for _ in range(3):
+                launch()
+            torch.cuda.synchronize()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(5)]
+            for a, b in evs:
+                a.record()
+                launch()
+                b.record()
+            torch.cuda.synchronize()
+            us = float(np.median([a.elapsed_time(b) for a, b in evs])) * 1e3
+            c = clocks.view(cus, 2).double().cpu()
+            ghz = float((c[:, 0] / (c[:, 1] / tick_hz)).median()) / 1e9
+            per_pair_us = us / (iters * wps)
+            rows.append({"variant": names[variant], "waves_per_simd": wps, "kernel_us": us,
+                         "us_per_pair_and_simd": per_pair_us, "cycles_per_pair_and_simd": per_pair_us * ghz * 1e3,
+                         "clock_ghz": ghz,
+                         "frac_of_2.5_pflops_if_nothing_else": PAIR_FLOP / (per_pair_us * 1e-6) * cus * 4 / 2.5e15})
+    best = min(r["us_per_pair_and_simd"] for r in rows if r["variant"] == names[3])
+    return {"metric": "issue floor of the attention tile loop: microseconds per block pair and SIMD", "value": best,
+            "unit": "us", "n_gpus": 1, "steps": 5, "warmup": 3, "ms_per_step": None, "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "mfma_mix: instruction-issue probes, operands in registers", "iters": iters, "cus": cus},
+            "rows": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c1", "c2", "c4", "c5", "ref_e2e", "stream", "overlap"])
+    ap.add_argument("--workload", default="c3", choices=["c3", "c1", "c2", "c4", "c5", "ref_e2e", "stream", "overlap", "mfma_mix"])
     ap.add_argument("--block-limit", type=int, default=1024, help="persistent workgroups of the balanced attention launch")
     ap.add_argument("--lpt-plan", action="store_true",
                     help="drive attention with the caller's LPT plan (the reference's balanced mode) instead of the kernel's own schedule")
@@ -755,6 +806,8 @@ def main():
         res = run_streaming(args)
     elif args.workload == "overlap":
         res = run_overlap(args)
+    elif args.workload == "mfma_mix":
+        res = run_issue_floor(args)
     else:
         res = run_membound_sweep(args)
     print(json.dumps(res))

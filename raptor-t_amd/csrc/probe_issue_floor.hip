@@ -3,7 +3,7 @@
 // in the way (every operand in registers, no memory access, no LDS, no barrier).
 //
 //   variant 0   the 32 v_mfma_f32_32x32x16_f16 of a pair alone (16 for K.Q^T, 16 for V^T.P^T)
-//   variant 1   + the 64 v_exp_f32 that turn a pair's 4096 scores into probabilities
+//   variant 1   + the 64 v_exp_f32 that turn a pair's 4096 scores into probabilities (and 32 v_xor that use them)
 //   variant 2   + the 32 v_cvt_pk_f16_f32 that round them to the matrix operand type
 //   variant 3   + the 32 packed additions of the row sums: the tile loop's whole mix, in the loop's own slot
 //               order (one matrix instruction, two exponentials, one conversion, one addition per slot)
@@ -28,8 +28,9 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define SB() __builtin_amdgcn_sched_barrier(0)
 
 template <int VARIANT>
-__global__ __launch_bounds__(512, 1) void issue_floor_kernel(float* out, int iters) {
+__global__ __launch_bounds__(512, 1) void issue_floor_kernel(float* out, long long* clocks, int iters) {
   const int lane = threadIdx.x & 63;
+  const long long c0 = clock64(), w0 = wall_clock64();
   f16x8 kf[8], vf[8], qf[2][4];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -58,28 +59,25 @@ __global__ __launch_bounds__(512, 1) void issue_floor_kernel(float* out, int ite
         SB();
         if ((i & 1) == 0) {
           const int c = i >> 1;
-          nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ktn * 4 + c], qf[ntn][c], c == 0 ? negm : nxt, 0, 0, 0);
+          // variant 0 keeps accumulating, so that no product of an earlier trip is dead code
+          nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ktn * 4 + c], qf[ntn][c], (c == 0 && VARIANT > 0) ? negm : nxt, 0, 0, 0);
         } else {
           const int tt = (i >> 1) & 1, s = i >> 2;
           o[tt][ntp] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[tt * 4 + 2 * ktp + s], pprev[s], o[tt][ntp], 0, 0, 0);
         }
         SB();
-        if (VARIANT >= 1) {
-          p[2 * i] = __builtin_amdgcn_exp2f(cur[2 * i]);
-          p[2 * i + 1] = __builtin_amdgcn_exp2f(cur[2 * i + 1]);
-        } else {
-          p[2 * i] = cur[2 * i];
-          p[2 * i + 1] = cur[2 * i + 1];
-        }
+        if (VARIANT == 0) continue;                     // the matrix instructions alone; P stays what it was
+        p[2 * i] = __builtin_amdgcn_exp2f(cur[2 * i]);
+        p[2 * i + 1] = __builtin_amdgcn_exp2f(cur[2 * i + 1]);
         if (VARIANT >= 2) {
           w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{p[2 * i], p[2 * i + 1]}, f16x2));
-        } else {
+        } else {                                        // the exponentials must be used by something: one full-rate instruction
           w[i] = __builtin_bit_cast(uint32_t, p[2 * i]) ^ __builtin_bit_cast(uint32_t, p[2 * i + 1]);
-          if (VARIANT == 0) w[i] = __builtin_bit_cast(uint32_t, cur[2 * i]);      // no vector work at all
         }
         if (VARIANT >= 3)
           lsum = __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, lsum) + __builtin_bit_cast(f16x2, w[i]));
       }
+      if (VARIANT == 0) continue;
       SB();
       u32x4 lo = {w[0], w[1], w[2], w[3]}, up = {w[4], w[5], w[6], w[7]};
       pb[S & 1][0] = __builtin_bit_cast(f16x8, lo);
@@ -91,21 +89,28 @@ __global__ __launch_bounds__(512, 1) void issue_floor_kernel(float* out, int ite
 #pragma unroll
   for (int e = 0; e < 16; ++e) s += o[0][0][e] + o[0][1][e] + o[1][0][e] + o[1][1][e] + sc[0][e] + sc[1][e];
   out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  // shader-clock cycles and ticks of the constant-rate clock this wave spent: their ratio is the clock the CU held
+  if (clocks && threadIdx.x == 0) {
+    clocks[2 * blockIdx.x] = clock64() - c0;
+    clocks[2 * blockIdx.x + 1] = wall_clock64() - w0;
+  }
 }
 
 }  // namespace
 
-// Launches one probe on `stream`: `out` needs cus * waves_per_simd * 256 floats of device memory.  Returns 0, or
-// -22 for an argument outside its range, -5 if the launch failed.
-extern "C" int rt_probe_issue_floor(int variant, int waves_per_simd, int iters, int cus, float* out, void* stream) {
+// Launches one probe on `stream`: `out` needs cus * waves_per_simd * 256 floats of device memory, `clocks` (optional)
+// 2 * cus 64-bit integers: per workgroup the shader-clock cycles and the constant-rate clock's ticks its first wave
+// ran for.  Returns 0, or -22 for an argument outside its range, -5 if the launch failed.
+extern "C" int rt_probe_issue_floor(int variant, int waves_per_simd, int iters, int cus, float* out, long long* clocks,
+                                    void* stream) {
   if (variant < 0 || variant > 3 || (waves_per_simd != 1 && waves_per_simd != 2) || iters < 1 || cus < 1 || !out) return -22;
   const dim3 grid(cus), block(256 * waves_per_simd);
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (variant) {
-    case 0: hipLaunchKernelGGL(issue_floor_kernel<0>, grid, block, 0, st, out, iters); break;
-    case 1: hipLaunchKernelGGL(issue_floor_kernel<1>, grid, block, 0, st, out, iters); break;
-    case 2: hipLaunchKernelGGL(issue_floor_kernel<2>, grid, block, 0, st, out, iters); break;
-    default: hipLaunchKernelGGL(issue_floor_kernel<3>, grid, block, 0, st, out, iters); break;
+    case 0: hipLaunchKernelGGL(issue_floor_kernel<0>, grid, block, 0, st, out, clocks, iters); break;
+    case 1: hipLaunchKernelGGL(issue_floor_kernel<1>, grid, block, 0, st, out, clocks, iters); break;
+    case 2: hipLaunchKernelGGL(issue_floor_kernel<2>, grid, block, 0, st, out, clocks, iters); break;
+    default: hipLaunchKernelGGL(issue_floor_kernel<3>, grid, block, 0, st, out, clocks, iters); break;
   }
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
