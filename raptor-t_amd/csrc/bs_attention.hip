@@ -293,32 +293,36 @@ __device__ inline float pair_sum(float x) {
 }
 
 // Writes the wave's 64x64 output tile, O^T[d = 32t + 8*(e>>2) + 4*(lane>>5) + (e&3)]
-// [query 32nt + (lane&31)] * w, to out[token][h*64 + d].  A lane holds 4 consecutive d of its query
-// per accumulator quad and its partner lane (lane ^ 32) the next 4: the two swap quads so that every
-// lane stores 16 bytes and the pair 32 consecutive bytes of the token's row.
+// [query 32nt + (lane&31)] * w, to out[token][h*64 + d], through the wave's own LDS room (64 rows, OUT_PITCH bytes
+// apart; no other wave touches it, and the LDS operations of one wave execute in order).  A lane holds 4
+// consecutive d of its query per accumulator quad: every lane parks its 16 quads, then lane L takes the 16-byte
+// chunk (L & 7) of tokens 8k + (L >> 3), so that a store instruction writes eight whole 128-byte lines.  Stores
+// straight from the accumulators (lane pairs swapping quads) write 32 bytes to each of 32 lines per instruction,
+// four pieces per line: same bits, 2-3 % more kernel time.
+constexpr int OUT_PITCH = 144;
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 template <typename T>
 __device__ inline void store_output(T* __restrict__ out_unit, int64_t row_stride, int lane, const State& st,
-                                    const float (&w)[2]) {
+                                    const float (&w)[2], char* stage) {
   const int l32 = lane & 31, hi = lane >> 5;
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) {
-    T* row = out_unit + int64_t(32 * nt + l32) * row_stride + (hi ? 0 : 8);
+    char* row = stage + (32 * nt + l32) * OUT_PITCH + 8 * hi;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int c4 = 0; c4 < 4; c4 += 2) {
-        uint32_t x[2], y[2];                                     // quads c4 and c4 + 1, rounded and packed
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          x[j] = Mma<T>::two(st.o[t][nt][4 * c4 + 2 * j] * w[nt], st.o[t][nt][4 * c4 + 2 * j + 1] * w[nt]);
-          y[j] = Mma<T>::two(st.o[t][nt][4 * c4 + 4 + 2 * j] * w[nt], st.o[t][nt][4 * c4 + 5 + 2 * j] * w[nt]);
-        }
-        // upper half of y <-> lower half of x: lower lanes end up with quad c4 + 1 of both lanes, upper lanes with quad c4
-        swap_halves(y[0], x[0]);
-        swap_halves(y[1], x[1]);
-        const u32x4 v = {y[0], y[1], x[0], x[1]};
-        *reinterpret_cast<u32x4*>(row + 32 * t + 8 * c4) = v;
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t x0 = Mma<T>::two(st.o[t][nt][4 * q] * w[nt], st.o[t][nt][4 * q + 1] * w[nt]);
+        const uint32_t x1 = Mma<T>::two(st.o[t][nt][4 * q + 2] * w[nt], st.o[t][nt][4 * q + 3] * w[nt]);
+        *reinterpret_cast<u32x2*>(row + 64 * t + 16 * q) = u32x2{x0, x1};
       }
+  }
+  const char* rd = stage + (lane >> 3) * OUT_PITCH + (lane & 7) * 16;
+  T* dst = out_unit + int64_t(lane >> 3) * row_stride + (lane & 7) * 8;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(rd + k * 8 * OUT_PITCH);
+    *reinterpret_cast<u32x4*>(dst + int64_t(8 * k) * row_stride) = v;
   }
 }
 
@@ -434,6 +438,7 @@ __device__ inline void request_q(const Args<T>& a, const Buffers<T>& b, const Un
 // query tile in row order (rows Q_STAGE_PITCH bytes apart).
 constexpr int Q_STAGE_PITCH = 144;
 constexpr int Q_STAGE_BYTES = 64 * Q_STAGE_PITCH;
+static_assert(OUT_PITCH == Q_STAGE_PITCH, "the output tile is parked in the room of the query tile");
 template <typename T> struct QSide { const T* bias; char* stage; };
 
 // Rows -> fragments through the wave's own LDS room (no other wave touches it: LDS operations of one wave
@@ -730,12 +735,12 @@ __device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const QSi
 
 // normalises the state and writes the unit's output tile
 template <typename T>
-__device__ inline void finish_unit(const Args<T>& a, const Unit& u, int lane, State& st) {
+__device__ inline void finish_unit(const Args<T>& a, const QSide<T>& qs, const Unit& u, int lane, State& st) {
   float w[2];
 #pragma unroll
   for (int nt = 0; nt < 2; ++nt) w[nt] = __builtin_amdgcn_rcpf(fmaxf(pair_sum(st.l[nt]), 1e-30f));
   const int64_t stride = int64_t(a.heads) * 64;
-  store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w);
+  store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w, qs.stage);
 }
 
 template <typename T>
@@ -758,7 +763,7 @@ __device__ inline bool run_solo(const Args<T>& a, const Buffers<T>& b, const QSi
     typename Mma<T>::v8 qf[2][4];
     slow_row<T, MASKED>(a, b, qbias, r, 0, 1, lane, false, qf, st);
   }
-  finish_unit<T>(a, u, lane, st);
+  finish_unit<T>(a, qbias, u, lane, st);
   return true;
 }
 
@@ -820,7 +825,8 @@ __device__ inline bool run_split4(const Args<T>& a, const Buffers<T>& b, const Q
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) w[nt] = __builtin_amdgcn_rcpf(fmaxf(st.l[nt], 1e-30f));
     const int64_t stride = int64_t(a.heads) * 64;
-    store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w);
+    // wave 0's room is the start of the park, which it has just finished reading
+    store_output<T>(a.out + int64_t(u.g0 + u.i) * 64 * stride + u.h * 64, stride, lane, st, w, qbias.stage);
   }
   __syncthreads();                                    // the park is read: the next item may stage its queries there
   return true;
@@ -854,41 +860,68 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const QSide<T> qbias{qbias_lds, reinterpret_cast<char*>(park) + wave * Q_STAGE_BYTES};
 
-  // geometry: prefix blocks, the list of rows that are not global rows, the sequences that have global rows
+  // Geometry: prefix blocks, the sequences that have global rows, the list of rows that are not global rows.  Every
+  // one of the 512 workgroups builds it for itself, so it is built by all 256 threads: sequence s's place in both
+  // lists follows from the number of sparse sequences before it (a ballot per wave, the waves' counts through LDS),
+  // since rows before s = blocks before s - 2 * (sparse sequences before s).
   int* const row_base = reinterpret_cast<int*>(park);            // per sequence: rows listed before it (scratch use of the park)
+  int* const wave_sparse = row_base + MAX_BATCH;                 // [round][wave]: sparse sequences among the wave's 64
   for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
   if (a.q_rows)
     for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias_lds[i] = a.q_bias[i];
   __syncthreads();
-  for (int i = threadIdx.x; i < a.batch; i += 256) {
-    int t = 64;
-    if (MASKED) {
-      t = a.seq_tokens[i] - 64 * (geo.sb[i + 1] - geo.sb[i] - 1);
-      t = t < 1 ? 1 : (t > 64 ? 64 : t);
-    }
-    geo.tail[i] = uint8_t(t);
-  }
-  if (threadIdx.x == 0) {
-    int rows = 0, sparse = 0;
-    for (int s = 0; s < a.batch; ++s) {
-      row_base[s] = rows;
-      const int n = geo.sb[s + 1] - geo.sb[s];
-      if (n >= RT_MIN_SPARSE_BLOCKS) {
-        geo.sparse_seq[sparse++] = uint16_t(s);
-        rows += n - 2;
-      } else {
-        rows += n;
+  const int rounds = (a.batch + 255) >> 8;                       // at most MAX_BATCH / 256 = 4
+  int before_in_wave[MAX_BATCH / 256];
+  bool is_sparse[MAX_BATCH / 256];
+#pragma unroll
+  for (int r = 0; r < MAX_BATCH / 256; ++r) {
+    before_in_wave[r] = 0;
+    is_sparse[r] = false;
+    if (r < rounds) {
+      const int sq = r * 256 + int(threadIdx.x);
+      is_sparse[r] = sq < a.batch && geo.sb[sq + 1] - geo.sb[sq] >= RT_MIN_SPARSE_BLOCKS;
+      const unsigned long long votes = __ballot(is_sparse[r]);
+      before_in_wave[r] = __popcll(votes & ((1ull << lane) - 1ull));
+      if (lane == 0) wave_sparse[r * 4 + wave] = __popcll(votes);
+      if (sq < a.batch) {
+        int t = 64;
+        if (MASKED) {
+          t = a.seq_tokens[sq] - 64 * (geo.sb[sq + 1] - geo.sb[sq] - 1);
+          t = t < 1 ? 1 : (t > 64 ? 64 : t);
+        }
+        geo.tail[sq] = uint8_t(t);
       }
     }
-    geo.n_rows = rows;
-    geo.n_sparse = sparse;
   }
   __syncthreads();
-  for (int g = threadIdx.x; g < a.nb_total; g += 256) {
-    const int s = upper_seq(geo.sb, a.batch, g);
-    const int n = geo.sb[s + 1] - geo.sb[s], i = g - geo.sb[s];
-    const bool sparse = n >= RT_MIN_SPARSE_BLOCKS;
-    if (!sparse || (i > 0 && i < n - 1)) geo.rows[row_base[s] + i - (sparse ? 1 : 0)] = uint32_t(s) << 16 | uint32_t(i);
+  {
+    int running = 0;                                             // sparse sequences before this wave's 64 of round r
+#pragma unroll
+    for (int r = 0; r < MAX_BATCH / 256; ++r)
+      if (r < rounds) {
+        int before = running;
+        for (int w = 0; w < 4; ++w) {
+          const int c = wave_sparse[r * 4 + w];
+          if (w < wave) before += c;
+          running += c;
+        }
+        const int sq = r * 256 + int(threadIdx.x);
+        if (sq < a.batch) {
+          const int k = before + before_in_wave[r];
+          row_base[sq] = geo.sb[sq] - 2 * k;
+          if (is_sparse[r]) geo.sparse_seq[k] = uint16_t(sq);
+        }
+      }
+    if (threadIdx.x == 0) {
+      geo.n_sparse = running;
+      geo.n_rows = geo.sb[a.batch] - 2 * running;
+    }
+  }
+  __syncthreads();
+  for (int sq = wave; sq < a.batch; sq += 4) {                   // a wave per sequence, a lane per row
+    const int n = geo.sb[sq + 1] - geo.sb[sq];
+    const int skip = n >= RT_MIN_SPARSE_BLOCKS ? 1 : 0;          // a sparse sequence's rows 0 and n - 1 are global rows
+    for (int i = skip + lane; i < n - skip; i += 64) geo.rows[row_base[sq] + i - skip] = uint32_t(sq) << 16 | uint32_t(i);
   }
   __syncthreads();
 
@@ -992,24 +1025,33 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       u.i = (ticket & 1) ? u.n - 1 : 0;
       return u;
     };
-    bool drained = false;
+    // The XCD's workgroup number w takes row w without asking; rows beyond the XCD's workgroups are drawn from the
+    // counter (ticket k = row wgs + k).  A batch with no more rows than workgroups touches no counter in this phase.
+    const int wgs = int(gridDim.x >> 3), wg_local = int(blockIdx.x >> 3);
+    const bool drawn_rows = n_glob > wgs;
+    int item = wg_local < n_glob ? wg_local : -1;
+    bool drained = item < 0 && !drawn_rows;
     while (!drained) {
       int n_rows_redo = 0;
       while (n_rows_redo < REDO_SLOTS) {
-        if (wave == 0) {
-          const int k = __builtin_amdgcn_readfirstlane(request_ticket(gq, lane));
-          if (lane == 0) s_item = k;
+        if (item < 0) {
+          if (!drawn_rows) { drained = true; break; }
+          if (wave == 0) {
+            const int k = __builtin_amdgcn_readfirstlane(request_ticket(gq, lane));
+            if (lane == 0) s_item = k;
+          }
+          __syncthreads();
+          item = wgs + s_item;
+          __syncthreads();
+          if (item >= n_glob) { drained = true; break; }
         }
-        __syncthreads();
-        const int item = s_item;
-        __syncthreads();
-        if (item >= n_glob) { drained = true; break; }
         bool ok = false;
         if (!MASKED) ok = run_split4<T, MASKED, true>(a, b, qbias, unit_of_row(item), lane, wave, park);
         if (!ok) {
           if (threadIdx.x == 0) redo_rows[n_rows_redo] = item;
           ++n_rows_redo;
         }
+        item = -1;
       }
       __syncthreads();
       for (int r = 0; r < n_rows_redo; ++r)
@@ -1047,7 +1089,6 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
     };
     const_int* pos_all = (const_int*)(uintptr_t)(a.to_pos);
     const int idx_total = pos_all[a.plan_heads * a.nb_total];       // entries in to_idx
-    const int waves_per_xcd = int(gridDim.x >> 3) * 4;
     int n_redo = 0;
     int item = item_of(request_ticket(uq, lane));
     int item_nx = item >= 0 ? item_of(request_ticket(uq, lane)) : -1;
@@ -1099,12 +1140,6 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
               nx.first_off = nx.goff + b0 * 8192;
             }
           }
-          // The unit after the next one.  Far from the end of the queue its ticket is drawn here, a
-          // whole tile loop before it is looked at; near the end only after the loop, so that a wave
-          // never sits on two waiting units while others run dry.  Both requests are always issued
-          // (one of them addresses nothing): no branch, so the waits further down count requests.
-          const bool far = has_next && hi - item_nx > 2 * waves_per_xcd;
-          const int t_early = request_ticket_if(uq, lane, far);
           int item_after = -1;
           primed = false;
           if (ok) {
@@ -1113,23 +1148,26 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
                          [&](int k) { t.qf[k >> 2][k & 3] = fetch_q<T>(b, qn, k); });
             lane = lane_id;
             asm volatile("" : "+v"(lane));
-            const int t_late = request_ticket_if(uq, lane, has_next && !far);
+            // The unit after the next one: its ticket is drawn here, behind the tile loop, and looked at once this
+            // unit's output is on its way.  (Drawn ahead of the loop, the request was still in flight at the loop's
+            // entry, where everything requested must have arrived: a device round trip of waiting per unit.)  The
+            // request is always issued (without a next unit it addresses nothing): no branch around it.
+            const int t_next = request_ticket_if(uq, lane, has_next);
             SB();
             primed = nx_short;
             if (sums_finite(st)) {
-              finish_unit<T>(a, cur.u, lane, st);
+              finish_unit<T>(a, qbias, cur.u, lane, st);
               SB();
-              item_after = has_next ? item_of(far ? t_early : t_late) : -1;
             } else {
               if (lane == 0) redo[wave][n_redo] = item;
               ++n_redo;
-              item_after = has_next ? item_of(far ? t_early : t_late) : -1;
             }
+            item_after = has_next ? item_of(t_next) : -1;
           } else {
             if (lane == 0) redo[wave][n_redo] = item;
             ++n_redo;
-            const int t_late = request_ticket_if(uq, lane, has_next && !far);
-            item_after = has_next ? item_of(far ? t_early : t_late) : -1;
+            const int t_next = request_ticket_if(uq, lane, has_next);
+            item_after = has_next ? item_of(t_next) : -1;
           }
           item = item_nx;
           item_nx = item_after;
