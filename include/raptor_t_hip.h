@@ -140,7 +140,9 @@ int rt_meta_check_to_index(const int* to_idx, const int* to_pos, int64_t idx_len
  * q (scaled by q_scale), k, vt in the head-major packed layout.  For rt_bs_attention_fwd
  * q_scale must be log2(e)/sqrt(64): the attention kernel evaluates the softmax in base 2.
  * q may be NULL: Q is then not written (a third less traffic), for rt_bs_attention_fwd_qrows,
- * which takes its queries from `qkv` itself. */
+ * which takes its queries from `qkv` itself.  bias may be NULL: the rows carry it already (the
+ * projection added it in its epilogue, rt_gemm_bt with RT_EPILOGUE_BIAS), and the kernel is a
+ * pure change of layout (plus the Q scale). */
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt,
                       const int* seq_blocks_dev, int batch, int total_blocks, int heads,
                       float q_scale, int dtype, void* stream);
@@ -193,7 +195,8 @@ int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, voi
  * k and vt still come from rt_qkv_bias_split (called with q = NULL).  Same stage of the
  * reference as rt_bs_attention_fwd; the reference always materialises Q
  * (layers/kernels/add_bias_and_transpose.cu:212-233).  seq_tokens_dev may be NULL.
- * At most 64 heads. */
+ * qkv_bias may be NULL when the rows carry the bias already (see rt_qkv_bias_split): only q_scale
+ * is applied.  At most 64 heads. */
 int rt_bs_attention_fwd_qrows(const void* qkv, const void* qkv_bias, float q_scale, const void* k,
                               const void* vt, void* out, const int* seq_blocks_dev,
                               const int* seq_tokens_dev, int batch, int total_blocks, int heads,

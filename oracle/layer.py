@@ -65,12 +65,20 @@ def _stored(x, store_dtype):
     return x if store_dtype is None else x.to(store_dtype).float()
 
 
-def attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block=64, store_dtype=None):
+def attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block=64, store_dtype=None,
+                       bias_in_projection=False):
     """QKV projection -> split -> block-sparse attention -> out-proj -> bias+residual+LN
-    (layers/multi_headed_attention.cpp:154-216)."""
+    (layers/multi_headed_attention.cpp:154-216).  bias_in_projection only matters with a store_dtype: the
+    projection's output is then stored once, with its bias (what a GEMM with a bias epilogue writes), instead of
+    being stored without it and again after the bias kernel, which is the reference's sequence."""
     st = lambda x: _stored(x, store_dtype)
-    qkv = st(hidden.float() @ w["qkv_weight"].float())
-    q, k, v = (st(x) for x in qkv_bias_split(qkv, w["qkv_bias"], heads))
+    if bias_in_projection:
+        rows = st(hidden.float() @ w["qkv_weight"].float() + w["qkv_bias"].float())
+        q, k, v = qkv_bias_split(rows, torch.zeros_like(w["qkv_bias"]), heads)
+        q = st(q)                                   # K and V are copies of what is stored; Q is scaled and stored again
+    else:
+        qkv = st(hidden.float() @ w["qkv_weight"].float())
+        q, k, v = (st(x) for x in qkv_bias_split(qkv, w["qkv_bias"], heads))
     ctx = st(attention.csr_attention(q, k, v, seq_blocks, to_idx, to_pos, plan_heads, block, scale=1.0))
     t = ctx.shape[0]
     proj = st(ctx.reshape(t, -1) @ w["attn_out_weight"].float())
@@ -78,12 +86,15 @@ def attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads,
                                       w["attn_ln_bias"], eps))
 
 
-def encoder_layer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps=1e-5, block=64, store_dtype=None):
+def encoder_layer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps=1e-5, block=64, store_dtype=None,
+                  bias_in_projection=False):
     """One layer: attention sub-layer, FFN up + GELU, FFN down + bias+residual+LN with the
     attention output as the residual (python/modeling_bert.py:172-210).  store_dtype: the dtype every tensor
-    that passes from one kernel to the next is rounded to (None: all fp32, the plain mathematical layer)."""
+    that passes from one kernel to the next is rounded to (None: all fp32, the plain mathematical layer);
+    bias_in_projection: see attention_sublayer."""
     st = lambda x: _stored(x, store_dtype)
-    attn = attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block, store_dtype)
+    attn = attention_sublayer(hidden, w, heads, seq_blocks, to_idx, to_pos, plan_heads, eps, block, store_dtype,
+                              bias_in_projection)
     inter = st(bias_gelu(attn @ w["inter_weight"].float(), w["inter_bias"]))
     out = st(inter @ w["out_weight"].float())
     return st(bias_residual_layernorm(out, attn, w["out_bias"], w["out_ln_weight"], w["out_ln_bias"], eps))

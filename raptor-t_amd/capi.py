@@ -231,7 +231,7 @@ def _attention_args(out, k, vt, seq_blocks_dev, heads, to_idx, to_pos, plan_head
 
 
 def qkv_bias_split(qkv, bias, q, k, vt, seq_blocks_dev, heads, q_scale):
-    """q may be None: Q is not written (for bs_attention_fwd_qrows)."""
+    """q may be None: Q is not written (for bs_attention_fwd_qrows).  bias may be None: the rows carry it already."""
     batch = seq_blocks_dev.numel() - 1
     if qkv.dim() != 2 or qkv.shape[0] % 64 or qkv.shape[1] != 3 * heads * 64:
         raise ValueError("qkv must be [tokens (a multiple of 64), 3 * heads * 64]")

@@ -457,9 +457,16 @@ __device__ inline void finish_q(const Args<T>& a, const QSide<T>& qs, const Unit
 #pragma unroll
     for (int k = 0; k < 8; ++k) qf[k >> 2][k & 3] = *reinterpret_cast<const v8*>(rd + (k >> 2) * 32 * Q_STAGE_PITCH + (k & 3) * 32);
   }
+  const bool with_bias = a.q_bias != nullptr;           // NULL: the projection's epilogue added the bias already
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    const v8 bb = *reinterpret_cast<const v8*>(qbias + u.h * 64 + c * 16 + (lane >> 5) * 8);
+    v8 bb;
+    if (with_bias) {
+      bb = *reinterpret_cast<const v8*>(qbias + u.h * 64 + c * 16 + (lane >> 5) * 8);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) bb[e] = static_cast<T>(0.f);
+    }
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -867,7 +874,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
   int* const row_base = reinterpret_cast<int*>(park);            // per sequence: rows listed before it (scratch use of the park)
   int* const wave_sparse = row_base + MAX_BATCH;                 // [round][wave]: sparse sequences among the wave's 64
   for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
-  if (a.q_rows)
+  if (a.q_rows && a.q_bias)
     for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias_lds[i] = a.q_bias[i];
   __syncthreads();
   const int rounds = (a.batch + 255) >> 8;                       // at most MAX_BATCH / 256 = 4
@@ -1245,7 +1252,7 @@ int launch_attention(const void* q, const void* q_rows, const void* q_bias, floa
                      void* out, const int* seq_blocks_dev, const int* seq_tokens_dev, int batch, int total_blocks,
                      int heads, const int* to_idx, const int* to_pos, int plan_heads, const int* from_idx,
                      const int* from_pos, int n_wg, int dtype, void* stream, int* own_queues = nullptr) {
-  RT_REQUIRE((q || (q_rows && q_bias)) && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE((q || q_rows) && k && vt && out && seq_blocks_dev && to_idx && to_pos, RT_EINVAL, "NULL pointer");
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1, RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d",
              batch, total_blocks, heads);
   RT_REQUIRE(plan_heads == 1 || plan_heads == heads, RT_EINVAL, "plan_heads=%d must be 1 or heads=%d", plan_heads, heads);
@@ -1317,7 +1324,7 @@ extern "C" int rt_bs_attention_fwd_qrows(const void* qkv, const void* qkv_bias, 
                                          const int* seq_tokens_dev, int batch, int total_blocks, int heads,
                                          const int* to_idx, const int* to_pos, int plan_heads, const int* from_idx,
                                          const int* from_pos, int n_wg, int dtype, void* stream) {
-  RT_REQUIRE(qkv && qkv_bias, RT_EINVAL, "NULL pointer");
+  RT_REQUIRE(qkv, RT_EINVAL, "NULL pointer");             // qkv_bias may be NULL: the rows carry the bias already
   return launch_attention(nullptr, qkv, qkv_bias, q_scale, k, vt, out, seq_blocks_dev, seq_tokens_dev, batch, total_blocks,
                           heads, to_idx, to_pos, plan_heads, from_idx, from_pos, n_wg, dtype, stream);
 }

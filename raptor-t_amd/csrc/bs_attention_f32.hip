@@ -106,7 +106,7 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
 #pragma unroll
       for (int s = 0; s < 16; ++s) {
         const int d = 4 * s + grp;
-        qreg[s] = (src[d] + a.q_bias[h * 64 + d]) * a.q_scale;
+        qreg[s] = (src[d] + (a.q_bias ? a.q_bias[h * 64 + d] : 0.f)) * a.q_scale;
       }
     } else {
       const float* src = a.q + head_base + int64_t(i) * 4096;

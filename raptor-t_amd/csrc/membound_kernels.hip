@@ -476,7 +476,12 @@ __global__ __launch_bounds__(256) void qkv_bias_split_kernel(const T* __restrict
 #pragma unroll
     for (int m = M0; m < 3; ++m) {
       Vec<T>::load(reinterpret_cast<const T*>(&raw[it][m]), x[m]);
-      Vec<T>::load(bias + m * dm + h * 64 + col, b[m]);
+      if (bias) {                               // NULL: the projection added it already (adding zero changes nothing)
+        Vec<T>::load(bias + m * dm + h * 64 + col, b[m]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) b[m][i] = 0.f;
+      }
     }
     // run `col8` (8 elements) of token `row` is lane (row & 31) + 32 * (col8 & 1) of fragment
     // 4 * (row >> 5) + (col8 >> 1); a 16-byte chunk of fp32 is half such a run
@@ -650,7 +655,7 @@ int rt_bias_gelu(void* out, const void* bias, int64_t rows, int width, int dtype
 
 int rt_qkv_bias_split(const void* qkv, const void* bias, void* q, void* k, void* vt, const int* seq_blocks_dev,
                       int batch, int total_blocks, int heads, float q_scale, int dtype, void* stream) {
-  RT_REQUIRE(qkv && bias && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");       // q may be NULL: not written
+  RT_REQUIRE(qkv && k && vt && seq_blocks_dev, RT_EINVAL, "NULL pointer");       // q may be NULL: not written; bias: none added
   RT_REQUIRE(batch >= 1 && total_blocks >= batch && heads >= 1 && int64_t(total_blocks) * heads < (int64_t(1) << 31),
              RT_EINVAL, "bad geometry: batch=%d total_blocks=%d heads=%d", batch, total_blocks, heads);
   RT_REQUIRE(dtype == RT_F16 || dtype == RT_BF16 || dtype == RT_F32, RT_EINVAL, "unknown dtype %d", dtype);

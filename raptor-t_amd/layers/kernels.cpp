@@ -222,6 +222,27 @@ void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b
                   current_stream()), name.c_str());
 }
 
+void MatMulBias(const torch::Tensor& A, const torch::Tensor& B, bool b_trans, const torch::Tensor& bias, torch::Tensor& out,
+                rt_gemm_ctx* handle, const std::string& name) {
+  require_cuda_contiguous(A, "A");
+  require_cuda_contiguous(B, "B");
+  require_cuda_contiguous(bias, "bias");
+  require_cuda_contiguous(out, "out");
+  if (A.dim() != 2 || B.dim() != 2) throw std::invalid_argument(name + ": operands must be matrices");
+  const int64_t n = b_trans ? B.size(0) : B.size(1);
+  if (A.size(1) != (b_trans ? B.size(1) : B.size(0)) || out.numel() != A.size(0) * n || bias.numel() != n ||
+      bias.scalar_type() != A.scalar_type() || B.scalar_type() != A.scalar_type() || out.scalar_type() != A.scalar_type())
+    throw std::invalid_argument(name + ": shape or dtype mismatch");
+  static std::map<std::string, float> no_info;
+  ScopedGpuTimer timer(no_info, "MatMul");
+  if (b_trans)
+    check(rt_gemm_bt(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), n, A.size(1),
+                     RT_EPILOGUE_BIAS, dtype_code(A), current_stream()), name.c_str());
+  else
+    check(rt_gemm_bias_act(handle, A.data_ptr(), B.data_ptr(), bias.data_ptr(), out.data_ptr(), A.size(0), n, A.size(1),
+                           RT_EPILOGUE_BIAS, dtype_code(A), current_stream()), name.c_str());
+}
+
 namespace {
 std::atomic<bool> g_epilogue_fusion{true};
 std::atomic<bool> g_q_from_rows{true};
@@ -273,7 +294,9 @@ double tune_layer_gemms(const std::vector<int64_t>& token_counts, int64_t hidden
   void* stream = current_stream();
   const int dt = dtype_code(a);
   for (int64_t m : token_counts) {
-    const int64_t shapes[4][3] = {{3 * hidden, hidden, RT_EPILOGUE_NONE}, {hidden, hidden, RT_EPILOGUE_NONE},
+    // the shapes and epilogues the layers run with the present switches
+    const int64_t qkv_epilogue = gemm_epilogue_fusion() ? RT_EPILOGUE_BIAS : RT_EPILOGUE_NONE;
+    const int64_t shapes[4][3] = {{3 * hidden, hidden, qkv_epilogue}, {hidden, hidden, RT_EPILOGUE_NONE},
                                   {ffn, hidden, RT_EPILOGUE_BIAS_GELU}, {hidden, ffn, RT_EPILOGUE_NONE}};
     for (const auto& sh : shapes)
       check(rt_gemm_bt(handle, a.data_ptr(), w.data_ptr(), sh[2] == RT_EPILOGUE_NONE ? nullptr : bias.data_ptr(),
@@ -296,7 +319,9 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
     const int64_t per_tensor = int64_t(block_num) * 64 * head_num * head_size;
     if (input_data.numel() != 3 * per_tensor)
       throw std::invalid_argument("add_bias_and_transpose_kernel: qkv must be [block_num * 64, 3 * heads * 64]");
-    require_data(bias, "qkv bias", dt, 3 * int64_t(head_num) * head_size);
+    // an undefined bias: the projection added it already (MatMulBias); only with kernel_fusion
+    if (bias.defined()) require_data(bias, "qkv bias", dt, 3 * int64_t(head_num) * head_size);
+    else if (!kernel_fusion) throw std::invalid_argument("add_bias_and_transpose_kernel: the unfused path needs the bias");
     if (!(kernel_fusion && attention_q_from_rows())) require_data(q, "q", dt, per_tensor);
     require_data(k, "k", dt, per_tensor);
     require_data(v, "v", dt, per_tensor);
@@ -306,7 +331,8 @@ void add_bias_and_transpose_kernel(const torch::Tensor& bias, torch::Tensor& inp
   // the attention kernel evaluates the softmax in base 2: fold log2(e) into the Q scale
   const float scale = kQScale;
   if (kernel_fusion) {
-    check(rt_qkv_bias_split(input_data.data_ptr(), bias.data_ptr(), attention_q_from_rows() ? nullptr : q.data_ptr(),
+    check(rt_qkv_bias_split(input_data.data_ptr(), bias.defined() ? bias.data_ptr() : nullptr,
+                            attention_q_from_rows() ? nullptr : q.data_ptr(),
                             k.data_ptr(), v.data_ptr(),
                             seq_len_info_tensor.data_ptr<int>(), batch_size, block_num, head_num, scale,
                             dtype_code(input_data), current_stream()), "rt_qkv_bias_split");
@@ -437,12 +463,13 @@ void sparse_attention(const torch::Tensor& q, const torch::Tensor& k, const torc
   }
   if (qkv_rows.defined()) {
     require_cuda_contiguous(qkv_rows, "qkv_rows");
-    require_cuda_contiguous(qkv_bias, "qkv_bias");
+    const bool with_bias = qkv_bias.defined();         // undefined: the rows carry the bias already
+    if (with_bias) require_cuda_contiguous(qkv_bias, "qkv_bias");
     if (qkv_rows.dim() != 2 || qkv_rows.size(0) != int64_t(block_num) * 64 || qkv_rows.size(1) != int64_t(head_num) * 192 ||
-        qkv_bias.numel() != qkv_rows.size(1) || qkv_rows.scalar_type() != out.scalar_type() ||
-        qkv_bias.scalar_type() != out.scalar_type())
+        qkv_rows.scalar_type() != out.scalar_type() ||
+        (with_bias && (qkv_bias.numel() != qkv_rows.size(1) || qkv_bias.scalar_type() != out.scalar_type())))
       throw std::invalid_argument("sparse_attention: qkv_rows must be [tokens, 3 * heads * 64] with a bias of that width");
-    check(rt_bs_attention_fwd_qrows(qkv_rows.data_ptr(), qkv_bias.data_ptr(), kQScale, k.data_ptr(), v.data_ptr(),
+    check(rt_bs_attention_fwd_qrows(qkv_rows.data_ptr(), with_bias ? qkv_bias.data_ptr() : nullptr, kQScale, k.data_ptr(), v.data_ptr(),
                                     out.data_ptr(), seq_len_info_tensor.data_ptr<int>(), tokens, batch_size, block_num,
                                     head_num, to_select_index, to_select_index_position, plan_heads, from_idx, from_pos,
                                     n_wg, dtype_code(out), current_stream()), "rt_bs_attention_fwd_qrows");

@@ -65,6 +65,12 @@ class ScopedGpuTimer {
 void MatMul(const torch::Tensor& A, bool a_trans, const torch::Tensor& B, bool b_trans, float alpha,
             torch::Tensor& out, float beta, rt_gemm_ctx* handle, const std::string& name);
 
+// MatMul with the bias add in the GEMM's epilogue: out[M,N] = A . B(^T) + bias[N], rounded once.  What the
+// reference does with MatMul followed by a bias kernel (layers/multi_headed_attention.cpp:154-175).  Times itself
+// under "MatMul".
+void MatMulBias(const torch::Tensor& A, const torch::Tensor& B, bool b_trans, const torch::Tensor& bias, torch::Tensor& out,
+                rt_gemm_ctx* handle, const std::string& name);
+
 // MatMul followed by add_bias_act_kernel, as one GEMM with the bias add and the tanh GELU in
 // its epilogue (what BertIntermediate's pair of calls, layers/bert_intermediate.cpp:22-30,
 // computes).  Times itself under "MatMul_bias_gelu".

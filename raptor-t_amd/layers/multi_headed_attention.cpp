@@ -51,11 +51,22 @@ std::pair<std::vector<int>, std::vector<int>> MultiHeadedAttention::GenerateSpar
   return {idx, pos};
 }
 
+bool MultiHeadedAttention::bias_in_projection(bool kernel_fusion) { return kernel_fusion && kernels::gemm_epilogue_fusion(); }
+
 void MultiHeadedAttention::FuseGemm012AddBIasTranspose(const torch::Tensor& input_tensor, torch::Tensor& q_out,
                                                        torch::Tensor& k_out, torch::Tensor& v_out,
                                                        torch::Tensor& seq_len_info_tensor, int total_seq_len, int d_num,
                                                        std::map<std::string, float>& info, bool kernel_fusion) const {
   torch::Tensor tmp_qkv_out1 = TensorSet::get_instance()->get_tensor("tmp_qkv_out1");
+  // With both fusions on, the projection adds its bias in the GEMM's epilogue (one rounding of the fp32 sum, no
+  // extra pass) and the split kernel only changes the layout: the bias it is handed is undefined.
+  if (bias_in_projection(kernel_fusion)) {
+    kernels::MatMulBias(input_tensor, qkv_weight_, true, qkv_bias_, tmp_qkv_out1, kernels::shared_gemm_handle(),
+                        "FuseGemm012AddBIasTranspose_MatMul");
+    kernels::add_bias_and_transpose_kernel(torch::Tensor(), tmp_qkv_out1, q_out, k_out, v_out, seq_len_info_tensor,
+                                           batch_size_, head_num_, block_num_, head_size_, info, kernel_fusion);
+    return;
+  }
   kernels::MatMul(input_tensor, false, qkv_weight_, true, 1, tmp_qkv_out1, 0, kernels::shared_gemm_handle(),
                   "FuseGemm012AddBIasTranspose_MatMul");
   kernels::add_bias_and_transpose_kernel(qkv_bias_, tmp_qkv_out1, q_out, k_out, v_out, seq_len_info_tensor, batch_size_,
@@ -115,7 +126,7 @@ void MultiHeadedAttention::operator()(const torch::Tensor& input_tensor, const t
                             from_select_index_tensor, from_select_index_position_tensor, to_idx, to_pos, plan_heads,
                             block_limit, block_num_, head_num_, info, balanced, attention_mask,
                             q_rows ? tensor_set->get_tensor("tmp_qkv_out1") : torch::Tensor(),
-                            q_rows ? qkv_bias_ : torch::Tensor());
+                            q_rows && !bias_in_projection(kernel_fusion) ? qkv_bias_ : torch::Tensor());
   semaphore->Release(layer_idx_, stream);
 
   kernels::MatMul(attention_out, false, dense_weight_, true, 1, output, 0, handle_, "Attention Output");

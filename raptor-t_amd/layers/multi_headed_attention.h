@@ -34,6 +34,9 @@ class MultiHeadedAttention {
   // batch on the calling thread and returns (to_select_index, to_select_index_position).
   std::pair<std::vector<int>, std::vector<int>> GenerateSparseBlockIndex() const;
 
+  // whether the QKV projection adds its bias in the GEMM's epilogue (both fusion switches on)
+  static bool bias_in_projection(bool kernel_fusion);
+
   void FuseGemm012AddBIasTranspose(const torch::Tensor& input_tensor, torch::Tensor& q_out, torch::Tensor& k_out,
                                    torch::Tensor& v_out, torch::Tensor& seq_len_info_tensor, int total_seq_len,
                                    int d_num, std::map<std::string, float>& info, bool kernel_fusion) const;

@@ -263,7 +263,7 @@ def test_attention_config3_full_size_properties(capi):
 def test_attention_queries_from_projection_rows(capi, dtype, n_wg, padded):
     """rt_bs_attention_fwd_qrows (queries read from the [T, 3*H*64] projection output, bias and scale applied on
     load; the split kernel called without a Q output) gives the same bits as the route through a materialised Q,
-    and both match the oracle."""
+    and both match the oracle; likewise with the bias already in the rows and none handed to either kernel."""
     say("attention qrows", dtype, n_wg, padded)
     heads, seq_lens = 4, [64 * 13, 64 * 3, 64 * 20, 64]
     t, dm = sum(seq_lens), heads * 64
@@ -293,8 +293,21 @@ def test_attention_queries_from_projection_rows(capi, dtype, n_wg, padded):
     kk, vv = (x[:, i * dm:(i + 1) * dm].to(dtype).view(t, heads, 64) for i in (1, 2))
     ref = oa.csr_attention(qs, kk, vv, sb.tolist(), idx, pos, ph, scale=1.0 / lh.LOG2E, seq_tokens=seq_tokens)
     assert (out_b.float().cpu() - ref).abs().max().item() <= 2e-2
-    with pytest.raises(capi.RaptorError):
-        capi.bs_attention_fwd_qrows(qkv, None, capi.Q_SCALE, k2, vt2, out_b, sb_d, heads, idx_d, pos_d, ph)
+    # rows that carry the bias already (what the projection's bias epilogue leaves), no bias handed over: the split
+    # kernel only changes the layout, the attention kernel only applies the scale; same bits as with the bias
+    # added by the kernels whenever row + bias is exact in the tensor type (here: the rows hold x + b rounded once)
+    rows = (qkv.float() + bias.float()).to(dtype)
+    zero = torch.zeros_like(bias)
+    q3, k3, vt3, k4, vt4 = new(), new(), new(), new(), new()
+    out_c, out_d = new().view(t, dm), new().view(t, dm)
+    capi.qkv_bias_split(rows, zero, q3, k3, vt3, sb_d, heads, capi.Q_SCALE)
+    capi.bs_attention_fwd(q3, k3, vt3, out_c, sb_d, heads, idx_d, pos_d, ph, from_idx, from_pos, tok_d)
+    capi.qkv_bias_split(rows, None, None, k4, vt4, sb_d, heads, capi.Q_SCALE)
+    capi.bs_attention_fwd_qrows(rows, None, capi.Q_SCALE, k4, vt4, out_d, sb_d, heads, idx_d, pos_d, ph, from_idx,
+                                from_pos, tok_d)
+    torch.cuda.synchronize()
+    assert torch.equal(k3, k4) and torch.equal(vt3, vt4) and torch.equal(out_c, out_d)
+    assert (out_d.float().cpu() - ref).abs().max().item() <= 2e-2
 
 
 def test_attention_maximum_batch(capi):

@@ -40,7 +40,7 @@ def say(*a):
 
 def _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype, max_pos=4096):
     """bf16: the oracle rounds every tensor that passes between two kernels to bf16, as the layer objects (and the
-    reference, in its fp16) store them; with 8 mantissa bits these roundings, not the kernels' arithmetic, decide
+    reference, in its fp16) store them (the projection's output once, with its bias: the layers' default route); with 8 mantissa bits these roundings, not the kernels' arithmetic, decide
     the distance to an all-fp32 layer (0.04 after two layers), and a bound that lets them through would hide a real
     error at small |y|.  fp16 is compared with the all-fp32 layer."""
     sb = md.seq_prefix_blocks(seq_lens)
@@ -49,7 +49,7 @@ def _oracle_encoder(x32, layers_w32, heads, seq_lens, eps, dtype, max_pos=4096):
     for li, w in enumerate(layers_w32):
         wr = {k: v.to(dtype).float() for k, v in w.items()}
         idx, pos = md.hf_to_index(seq_lens, li, heads, max_pos=max_pos)
-        h = ol.encoder_layer(h, wr, heads, sb, idx, pos, heads, eps, store_dtype=store)
+        h = ol.encoder_layer(h, wr, heads, sb, idx, pos, heads, eps, store_dtype=store, bias_in_projection=True)
     return h
 
 
@@ -689,7 +689,7 @@ def test_large_workload_matches_oracle_layer_by_layer(pkg, mb, ut):
     for li in range(layers):
         x_in = x0[rows].to(dt).float() if li == 0 else kept[li - 1]
         idx, pos = md.hf_to_index([seq_lens[s]], li, heads, max_pos=max_pos)
-        want = ol.encoder_layer(x_in, w32[li], heads, sb, idx, pos, heads, 1e-5, store_dtype=dt)
+        want = ol.encoder_layer(x_in, w32[li], heads, sb, idx, pos, heads, 1e-5, store_dtype=dt, bias_in_projection=True)
         stats.append(lh.outliers(kept[li], want, dt, k=2.0) + ((kept[li] - want).abs().max().item(),))
     say("  per layer (share outside the per-element bound, worst in ulp of the row maximum, rms, max abs):")
     for li, st in enumerate(stats):

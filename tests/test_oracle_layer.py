@@ -129,3 +129,10 @@ def test_stored_tensors_option_rounds_between_kernels_only():
     assert torch.equal(rounded, rounded.to(torch.bfloat16).float())
     err = (rounded - plain).abs().max().item()
     assert 0 < err <= 0.1, err
+    # the projection stored once, with its bias: the plain layer in fp32 (the sum of two fp32 roundings apart),
+    # another set of bf16 roundings (not the same values, the same size of error) in bf16
+    same = ol.encoder_layer(x, w, heads, sb, idx, pos, heads, store_dtype=torch.float32, bias_in_projection=True)
+    assert (plain - same).abs().max().item() <= 1e-5
+    once = ol.encoder_layer(x, w, heads, sb, idx, pos, heads, store_dtype=torch.bfloat16, bias_in_projection=True)
+    assert torch.equal(once, once.to(torch.bfloat16).float()) and not torch.equal(once, rounded)
+    assert 0 < (once - plain).abs().max().item() <= 0.1
