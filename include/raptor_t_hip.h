@@ -96,6 +96,14 @@ int rt_meta_seq_prefix_blocks(const int* seq_lens, int batch, int* out_seq_block
  * replaces python/modeling_big_bird.py:573-597 with :1039-1314. */
 int rt_meta_rand_attn(int length, uint32_t seed, int heads, int max_pos, int policy, int* out);
 
+/* The plans rt_meta_rand_attn / rt_meta_build_to_index (RT_PLAN_HF) draw are pure functions of (length, seed, heads,
+ * max_pos, policy); the library keeps the ones it has drawn in a memo table (the oracle's own code,
+ * python/modeling_big_bird.py:573-597, draws them again for every forward pass: 2 ms per layer of a 16-sequence
+ * batch, which a worker thread otherwise spends per batch).  max_bytes >= 0 sets the table's bound (0: keep
+ * nothing, and forget what is kept; default 64 MiB), max_bytes < 0 leaves it; hits / misses (may be NULL) receive
+ * the look-up counts so far.  No counterpart in the reference. */
+int rt_meta_set_plan_cache(int64_t max_bytes, int64_t* hits, int64_t* misses);
+
 /* Sizes of the CSR that rt_meta_build_to_index will write. */
 int rt_meta_to_index_size(const int* seq_blocks, int batch, int plan_heads,
                           int64_t* idx_len, int64_t* pos_len);

@@ -21,7 +21,7 @@ RT_GEMM_TUNE_ALL = -1
 
 EXPORTS = [
     "rt_last_error_string", "rt_abi_version", "rt_time_next_launch", "rt_meta_np_permutations", "rt_meta_seq_prefix_blocks",
-    "rt_meta_rand_attn", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
+    "rt_meta_rand_attn", "rt_meta_set_plan_cache", "rt_meta_to_index_size", "rt_meta_build_to_index", "rt_meta_block_costs",
     "rt_meta_partition_lpt", "rt_meta_check_partition", "rt_meta_check_to_index", "rt_qkv_bias_split", "rt_unpack_head_tiles", "rt_bs_attention_fwd",
     "rt_bs_attention_fwd_masked", "rt_bs_attention_fwd_qrows", "rt_bs_attention_fwd_no_alloc",
     "rt_bias_residual_layernorm", "rt_bias_gelu", "rt_embed_layernorm", "rt_gemm_create", "rt_gemm_destroy", "rt_gemm_set_tuning", "rt_gemm_set_retuning", "rt_gemm",
@@ -55,6 +55,7 @@ def lib():
         L.rt_meta_seq_prefix_blocks.argtypes = [i32p, I, i32p]
         L.rt_meta_rand_attn.argtypes = [I, U, I, I, I, i32p]
         L.rt_meta_to_index_size.argtypes = [i32p, I, I, i64p, i64p]
+        L.rt_meta_set_plan_cache.argtypes = [L64, i64p, i64p]
         L.rt_meta_build_to_index.argtypes = [i32p, I, I, I, U, I, I, i32p, i32p, L64, i32p, L64]
         L.rt_meta_block_costs.argtypes = [i32p, I, i32p, i64p]
         L.rt_meta_partition_lpt.argtypes = [i32p, I, I, I, i32p, i32p]
@@ -122,6 +123,13 @@ def rand_attn(length, seed, heads, max_pos=4096, policy=RT_POLICY_REFERENCE_PATC
     out = np.empty((heads, n - 2, 3), dtype=np.int32)
     check(lib().rt_meta_rand_attn(length, seed, heads, max_pos, policy, _p(out)))
     return out
+
+
+def plan_cache(max_bytes=-1):
+    """Sets the bound of the library's memo table of plans (negative: leave it) and returns (hits, misses) so far."""
+    h, m = ctypes.c_int64(), ctypes.c_int64()
+    check(lib().rt_meta_set_plan_cache(max_bytes, ctypes.byref(h), ctypes.byref(m)))
+    return h.value, m.value
 
 
 def to_index_size(seq_blocks, plan_heads):

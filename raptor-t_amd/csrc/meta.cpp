@@ -8,7 +8,11 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
 #include <queue>
+#include <tuple>
 #include <vector>
 
 #include "rt_common.h"
@@ -113,7 +117,9 @@ static void max_plan_one_head(NpRng& rng, int max_pos, int last_idx, int rows_wa
 // First `want` legal blocks of a permutation of [to_start, to_end):
 // python/modeling_big_bird.py:1261-1314.
 static std::vector<int> single_row(NpRng& rng, int block_id, int to_start, int to_end, int want) {
-  std::vector<int> perm = iota_range(to_start, to_end);
+  static thread_local std::vector<int> perm;           // called once per row and head: no allocation per call
+  perm.clear();
+  for (int x = to_start; x < to_end; ++x) perm.push_back(x);
   rng.permute(perm);
   auto illegal = [&](int b) {
     if (b >= block_id - 1 && b <= block_id + 1) return true;
@@ -185,7 +191,50 @@ static bool uses_max_plan(int length, int policy) {
   return length % 256 == 0 && length >= 1024;      // python/modeling_big_bird.py:574, from 1024 up
 }
 
+static int rand_attn_compute(int length, uint32_t seed, int heads, int max_pos, int policy, int* out);
+
+// Memo table of the plans: a plan is a pure function of (length, seed, heads, max_pos, policy), and drawing one
+// costs as many generator steps as the oracle's numpy code (0.1-0.2 ms for a 4096-token sequence of 12 heads), which
+// a server would otherwise repeat for every batch and layer.  Bounded by bytes; when full, nothing more is kept.
+namespace {
+typedef std::tuple<int, uint32_t, int, int, int> PlanKey;
+struct PlanCache {
+  std::mutex m;
+  std::map<PlanKey, std::shared_ptr<const std::vector<int>>> plans;
+  int64_t bytes = 0, limit = int64_t(64) << 20, hits = 0, misses = 0;
+};
+PlanCache& plan_cache() { static PlanCache c; return c; }
+}  // namespace
+
 static int rand_attn_impl(int length, uint32_t seed, int heads, int max_pos, int policy, int* out) {
+  PlanCache& c = plan_cache();
+  const PlanKey key(length, seed, heads, max_pos, policy);
+  const size_t cnt = size_t(heads) * size_t(length / RT_BLOCK - 2) * RT_NUM_RAND;
+  {
+    std::lock_guard<std::mutex> lk(c.m);
+    if (c.limit > 0) {
+      auto it = c.plans.find(key);
+      if (it != c.plans.end()) {
+        ++c.hits;
+        std::shared_ptr<const std::vector<int>> plan = it->second;
+        std::copy(plan->begin(), plan->end(), out);
+        return RT_OK;
+      }
+      ++c.misses;
+    }
+  }
+  const int rc = rand_attn_compute(length, seed, heads, max_pos, policy, out);
+  if (rc != RT_OK) return rc;
+  std::lock_guard<std::mutex> lk(c.m);
+  const int64_t add = int64_t(cnt) * int64_t(sizeof(int)) + 64;
+  if (c.limit > 0 && c.bytes + add <= c.limit && !c.plans.count(key)) {
+    c.plans[key] = std::make_shared<const std::vector<int>>(out, out + cnt);
+    c.bytes += add;
+  }
+  return RT_OK;
+}
+
+static int rand_attn_compute(int length, uint32_t seed, int heads, int max_pos, int policy, int* out) {
   const int nb = length / RT_BLOCK;
   NpRng rng(seed);
   if (uses_max_plan(length, policy)) {
@@ -270,6 +319,18 @@ int rt_meta_rand_attn(int length, uint32_t seed, int heads, int max_pos, int pol
              "length %d: block-sparse plans exist from %d tokens, multiples of %d", length,
              RT_MIN_SPARSE_BLOCKS * RT_BLOCK, RT_BLOCK);
   return rand_attn_impl(length, seed, heads, max_pos, policy, out);
+}
+
+int rt_meta_set_plan_cache(int64_t max_bytes, int64_t* hits, int64_t* misses) {
+  PlanCache& c = plan_cache();
+  std::lock_guard<std::mutex> lk(c.m);
+  if (hits) *hits = c.hits;
+  if (misses) *misses = c.misses;
+  if (max_bytes >= 0) {
+    c.limit = max_bytes;
+    if (c.bytes > c.limit) { c.plans.clear(); c.bytes = 0; }
+  }
+  return RT_OK;
 }
 
 int rt_meta_to_index_size(const int* sb, int batch, int plan_heads, int64_t* idx_len, int64_t* pos_len) {

@@ -1,6 +1,6 @@
 // Metadata / stream pipeline: one worker thread per encoder layer builds that layer's
 // to-block CSR as soon as a batch is published, stages it in pinned memory, copies it
-// on a private copy stream and records an event the compute stream later waits on.
+// (a small kernel on a private stream) and records an event the compute stream later waits on.
 //
 // Replaces, from the reference: the per-layer counting semaphore
 // (layers/semaphore.cpp:8-37), MetaData::update_meta_data / terminate_thread
@@ -76,6 +76,16 @@ struct rt_pipeline {
 };
 
 namespace {
+
+// Copies a CSR from pinned host memory (mapped into the device's address space) to its device buffers.
+constexpr int UPLOAD_BLOCKS = 32;
+__global__ __launch_bounds__(256) void upload_csr_kernel(const int* __restrict__ host_idx, int* __restrict__ dev_idx,
+                                                         int64_t n_idx, const int* __restrict__ host_pos,
+                                                         int* __restrict__ dev_pos, int64_t n_pos) {
+  const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n_idx; i += stride) dev_idx[i] = host_idx[i];
+  for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n_pos; i += stride) dev_pos[i] = host_pos[i];
+}
 
 int plan_heads_of(const rt_pipeline* p) { return p->plan_mode == RT_PLAN_REFERENCE ? 1 : p->heads; }
 
@@ -165,8 +175,13 @@ int build_layer(rt_pipeline* p, int l, int64_t gen, const std::vector<int>& sb) 
     if (rc) return rc;
   }
   if (p->device >= 0) {
-    HIP_TRY(hipMemcpyAsync(s.dev_idx, s.host_idx, need_idx * sizeof(int), hipMemcpyHostToDevice, L.copy_stream));
-    HIP_TRY(hipMemcpyAsync(s.dev_pos, s.host_pos, need_pos * sizeof(int), hipMemcpyHostToDevice, L.copy_stream));
+    // A kernel that reads the pinned buffers, not hipMemcpyAsync: a copy engine cannot wait for work on its own, so
+    // the runtime makes the calling thread wait for whatever the stream's hardware queue still holds (the 13 streams
+    // of a 12-layer pipeline share 4 hardware queues with the compute stream), which stalled workers for a whole
+    // step's kernels.  A kernel launch never waits on the host.
+    hipLaunchKernelGGL(upload_csr_kernel, dim3(UPLOAD_BLOCKS), dim3(256), 0, L.copy_stream, s.host_idx, s.dev_idx,
+                       need_idx, s.host_pos, s.dev_pos, need_pos);
+    HIP_TRY(hipGetLastError());
     HIP_TRY(hipEventRecord(s.copied, L.copy_stream));
   }
   return RT_OK;

@@ -112,6 +112,15 @@ PYBIND11_MODULE(raptor_t, m) {
            py::arg("head_num"), py::arg("balanced") = false);
   }
 
+  m.def("plan_cache",
+        [](int64_t max_bytes) {
+          int64_t hits = 0, misses = 0;
+          if (rt_meta_set_plan_cache(max_bytes, &hits, &misses) != RT_OK) throw std::runtime_error(rt_last_error_string());
+          return std::make_pair(hits, misses);
+        },
+        py::arg("max_bytes") = -1,
+        "Bound in bytes of the memo table of random-block plans the index workers draw from (0: keep nothing; negative: "
+        "leave it as it is).  Returns (hits, misses) so far.");
   m.def("set_micro_batch_lane", &layers::set_current_lane, py::arg("lane"),
         "Selects which of the two independent sets of per-batch state (scratch tensors, published geometry, block-index "
         "pipeline, GEMM workspace) the following calls use: a caller that keeps two micro-batches in flight on two "

@@ -139,6 +139,34 @@ def test_launch_event_pair_is_per_thread_and_withdrawable(capi):
     assert capi.time_next_launch(None, None) == 0
 
 
+def test_plan_memo_table_returns_what_a_fresh_draw_returns(capi):
+    """The memo table of plans changes nothing but the time: every index built with it equals the index built with
+    the table off, for both plan families, several seeds and position counts; look-ups are counted; a bound of zero
+    forgets everything."""
+    lens = [832, 1024, 64, 2048, 1088, 4096, 1024]
+    sb = capi.seq_prefix_blocks(lens)
+    try:
+        capi.plan_cache(0)
+        fresh = {(seed, mp): capi.build_to_index(sb, 3, seed=seed, max_pos=mp) for seed in (0, 5) for mp in (4096, 8192)}
+        capi.plan_cache(1 << 20)
+        h0, m0 = capi.plan_cache()
+        for rnd in range(2):
+            for (seed, mp), (idx, pos) in fresh.items():
+                got_idx, got_pos = capi.build_to_index(sb, 3, seed=seed, max_pos=mp)
+                assert np.array_equal(got_idx, idx) and np.array_equal(got_pos, pos)
+        h1, m1 = capi.plan_cache()
+        sparse = sum(1 for n in lens if n >= 768)
+        assert m1 - m0 == 4 * (sparse - 1)                   # the two 1024-token sequences share a plan
+        assert h1 - h0 == 4 * (sparse + 1)
+        assert np.array_equal(capi.rand_attn(1088, 5, 3), capi.rand_attn(1088, 5, 3))
+        capi.plan_cache(0)                                    # forget, then a tiny bound: nothing fits, results unchanged
+        capi.plan_cache(16)
+        idx, pos = capi.build_to_index(sb, 3, seed=0, max_pos=4096)
+        assert np.array_equal(idx, fresh[(0, 4096)][0])
+    finally:
+        capi.plan_cache(64 << 20)
+
+
 def _host_csr(ptr, n):
     return np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(ctypes.c_int)), shape=(n,)).copy()
 
