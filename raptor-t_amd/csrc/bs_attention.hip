@@ -457,16 +457,9 @@ __device__ inline void finish_q(const Args<T>& a, const QSide<T>& qs, const Unit
 #pragma unroll
     for (int k = 0; k < 8; ++k) qf[k >> 2][k & 3] = *reinterpret_cast<const v8*>(rd + (k >> 2) * 32 * Q_STAGE_PITCH + (k & 3) * 32);
   }
-  const bool with_bias = a.q_bias != nullptr;           // NULL: the projection's epilogue added the bias already
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    v8 bb;
-    if (with_bias) {
-      bb = *reinterpret_cast<const v8*>(qbias + u.h * 64 + c * 16 + (lane >> 5) * 8);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) bb[e] = static_cast<T>(0.f);
-    }
+    const v8 bb = *reinterpret_cast<const v8*>(qbias + u.h * 64 + c * 16 + (lane >> 5) * 8);
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
@@ -874,8 +867,8 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
   int* const row_base = reinterpret_cast<int*>(park);            // per sequence: rows listed before it (scratch use of the park)
   int* const wave_sparse = row_base + MAX_BATCH;                 // [round][wave]: sparse sequences among the wave's 64
   for (int i = threadIdx.x; i <= a.batch; i += 256) geo.sb[i] = a.seq_blocks[i];
-  if (a.q_rows && a.q_bias)
-    for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias_lds[i] = a.q_bias[i];
+  if (a.q_rows)                                                  // without a bias (the rows carry it already): zeros
+    for (int i = threadIdx.x; i < a.heads * 64; i += 256) qbias_lds[i] = a.q_bias ? a.q_bias[i] : static_cast<T>(0.f);
   __syncthreads();
   const int rounds = (a.batch + 255) >> 8;                       // at most MAX_BATCH / 256 = 4
   int before_in_wave[MAX_BATCH / 256];
