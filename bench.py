@@ -41,11 +41,30 @@ def block_pairs(seq_blocks, heads):
     return tot * heads
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default workload and scaled by
-# what the same counters read for the QKV split kernel (a copy of known size); the summaries and the commands are
-# in profiles/memory_kernels_c3_traffic.txt.  Only valid for that workload.
-MEASURED_TRAFFIC_C3 = {"bs_attention_kernel": 518.2e6, "bias_residual_layernorm_kernel": 171.4e6,
-                       "bias_gelu_kernel": 457.0e6, "qkv_bias_split_kernel_q": 342.8e6, "qkv_bias_split_kernel": 228.5e6}
+TRAFFIC_PROFILE = os.path.join("profiles", "memory_kernels_c3_traffic.txt")
+
+
+def measured_traffic_c3():
+    """HBM-side bytes per launch of the hand-written kernels at the default workload, read from the `total MB` column
+    of the table in profiles/memory_kernels_c3_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by
+    what the same counters read for the K/V split kernel, a copy of known size; the commands are in that file).
+    Only valid for that workload and the kernels the profile was taken with; {} if the file is not there."""
+    keys = {"qkv_bias_split_kernel<__half,false>": "qkv_bias_split_kernel", "qkv_bias_split_kernel<__half,true>": "qkv_bias_split_kernel_q",
+            "bias_gelu_kernel<__half>": "bias_gelu_kernel", "bias_residual_layernorm_kernel<...>": "bias_residual_layernorm_kernel",
+            "bs_attention_kernel<_Float16,": "bs_attention_kernel"}
+    out = {}
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            for line in f:
+                tok = line.split()
+                for name, key in keys.items():
+                    if tok and tok[0] == name:
+                        nums = [t for t in tok[1:] if t.replace(".", "", 1).isdigit()]
+                        if len(nums) >= 7:                      # FETCH raw, WRITE raw, read, written, total, algorithmic, ratio
+                            out[key] = float(nums[4]) * 1e6
+    except OSError:
+        pass
+    return out
 
 
 def hbm_roofline(name, bytes_per_launch, us_per_launch, traffic=None):
@@ -298,7 +317,7 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
     att_flops = pairs * PAIR_FLOP
     ach = att_flops / (att_us * 1e-6)
     sz = 4 if dtype == "f32" else 2
-    traffic = MEASURED_TRAFFIC_C3 if name.startswith("c3") else {}
+    traffic = measured_traffic_c3() if name.startswith("c3") else {}
     out = {
         "metric": METRIC, "value": len(seq_lens) / (elapsed / args.steps), "unit": "seqs/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step, "ms_per_layer": ms_step / layers,
@@ -311,7 +330,8 @@ def run_encoder(args, name, hidden, heads, ffn, layers, dtype, seq_lens, max_pos
                    "weights": "random N(0,0.02)", "plan": "per-head HF plan, seed = layer index"},
         "roofline": {"kernel": "bs_attention_kernel", "bound": "mfma", "achieved": ach / 1e12,
                      "peak": MFMA_PEAK[dtype] / 1e12, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK[dtype],
-                     "traffic": traffic.get("bs_attention_kernel"), "flop_per_launch": att_flops,
+                     "traffic": traffic.get("bs_attention_kernel"),
+                     "traffic_source": TRAFFIC_PROFILE if traffic.get("bs_attention_kernel") else None, "flop_per_launch": att_flops,
                      "block_pairs": pairs, "us_per_launch": att_us, "algorithmic_hbm_bytes": 4 * t * hidden * sz},
         "roofline_layernorm": hbm_roofline("bias_residual_layernorm_kernel", 3 * t * hidden * sz,
                                            per["add_bias_and_layernorm_kernel"],
@@ -427,24 +447,32 @@ def run_membound_sweep(args):
         def fn():
             state[0] = (state[0] + 1) % len(sets)
             call(*sets[state[0]])
-        cold = time_kernel(fn, args.steps, args.warmup)
-        warm = time_kernel(lambda: call(*sets[0]), args.steps, args.warmup)
+        # --sweep-mode restricts the run to one timing mode (for counter runs, where the two must not mix)
+        cold = time_kernel(fn, args.steps, args.warmup) if args.sweep_mode in ("both", "rotating") else float("nan")
+        warm = time_kernel(lambda: call(*sets[0]), args.steps, args.warmup) if args.sweep_mode in ("both", "resident") else float("nan")
         for st in sets:
             assert bool(torch.isfinite(st[0]).all()), "output is not finite"
         return cold, warm
 
+    kernels = set(args.sweep_kernels.split(","))
     for dt, name in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
-        for t in (8192, 32768, 65536):
+        if name not in args.sweep_dtypes.split(","):
+            continue
+        for t in [int(x) for x in args.sweep_rows.split(",")]:
             g = torch.Generator(device="cuda").manual_seed(0)
             rn = lambda *s: torch.randn(*s, generator=g, device="cuda").to(dt)
             b, ga, be, b2 = rn(768), rn(768), rn(768), rn(3072)
-            us, warm = rotating(lambda: (rn(t, 768), rn(t, 768)),
-                                lambda x, r: capi.bias_residual_layernorm(x, r, b, ga, be, 1e-5), 2 * t * 768 * 2)
-            rows.append(dict(hbm_roofline("bias_residual_layernorm_kernel", 3 * t * 768 * 2, us), tokens=t, dtype=name, us=us,
-                             us_resident=warm, frac_resident=3 * t * 768 * 2 / (warm * 1e-6) / HBM_PEAK))
-            us, warm = rotating(lambda: (rn(t, 3072),), lambda y: capi.bias_gelu(y, b2), t * 3072 * 2)
-            rows.append(dict(hbm_roofline("bias_gelu_kernel", 2 * t * 3072 * 2, us), tokens=t, dtype=name, us=us,
-                             us_resident=warm, frac_resident=2 * t * 3072 * 2 / (warm * 1e-6) / HBM_PEAK))
+            if "ln" in kernels:
+                us, warm = rotating(lambda: (rn(t, 768), rn(t, 768)),
+                                    lambda x, r: capi.bias_residual_layernorm(x, r, b, ga, be, 1e-5), 2 * t * 768 * 2)
+                rows.append(dict(hbm_roofline("bias_residual_layernorm_kernel", 3 * t * 768 * 2, us), tokens=t, dtype=name, us=us,
+                                 us_resident=warm, frac_resident=3 * t * 768 * 2 / (warm * 1e-6) / HBM_PEAK))
+            if "gelu" in kernels:
+                us, warm = rotating(lambda: (rn(t, 3072),), lambda y: capi.bias_gelu(y, b2), t * 3072 * 2)
+                rows.append(dict(hbm_roofline("bias_gelu_kernel", 2 * t * 3072 * 2, us), tokens=t, dtype=name, us=us,
+                                 us_resident=warm, frac_resident=2 * t * 3072 * 2 / (warm * 1e-6) / HBM_PEAK))
+            if "embed" not in kernels:
+                continue
             # packed-input front end: fp32 tables (BigBird vocabulary 50358, 4096 positions), output in dt; per
             # token one fp32 word row read and one output row written (position / type rows recur and stay cached)
             gi = torch.Generator().manual_seed(0)
@@ -458,7 +486,9 @@ def run_membound_sweep(args):
                                 t * 768 * (4 + 2))
             rows.append(dict(hbm_roofline("embed_layernorm_kernel", t * 768 * (4 + 2), us), tokens=t, dtype=name, us=us,
                              us_resident=warm, frac_resident=t * 768 * (4 + 2) / (warm * 1e-6) / HBM_PEAK))
-    best_ln = max(r["frac"] for r in rows if r["kernel"].startswith("bias_residual"))
+    ln_rows = [r for r in rows if r["kernel"].startswith("bias_residual")]
+    ln_fracs = [r["frac"] for r in ln_rows if r["frac"] == r["frac"]] or [r["frac_resident"] for r in ln_rows]
+    best_ln = max(ln_fracs) if ln_fracs else float("nan")
     res = {"metric": "fused add-bias+LayerNorm / bias+GELU achieved HBM GB/s", "value": best_ln * 8000.0, "unit": "GB/s",
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "f16/bf16", "data": "synthetic",
@@ -779,6 +809,11 @@ def main():
     ap.add_argument("--no-pretune", action="store_true",
                     help="stream workload: skip the start-up GEMM tuning over the range of token counts")
     ap.add_argument("--no-two-streams", action="store_true", help="skip the two-stream comparison after the timed steps")
+    ap.add_argument("--sweep-rows", default="8192,32768,65536", help="c4: token counts of the sweep")
+    ap.add_argument("--sweep-kernels", default="ln,gelu,embed", help="c4: which of ln, gelu, embed to run")
+    ap.add_argument("--sweep-dtypes", default="f16,bf16", help="c4: which of f16, bf16 to run")
+    ap.add_argument("--sweep-mode", default="both", choices=["both", "rotating", "resident"],
+                    help="c4: time launches on buffers in rotation, on one buffer, or both")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=2)
     args = ap.parse_args()

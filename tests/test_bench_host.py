@@ -64,3 +64,16 @@ def test_cpu_baseline_helpers():
     assert runs == 3 and len(calls) == 5 and med >= 0.0
     med, runs = b.timed_median(lambda: None, warmup=0, reps=4, budget_s=60.0)
     assert runs == 4
+
+
+def test_traffic_figures_come_from_the_committed_profile():
+    """bench.py's `traffic` fields are read from the table of profiles/memory_kernels_c3_traffic.txt: every
+    hand-written kernel of the default line has a row, the memory-bound ones at their algorithmic bytes."""
+    b = _bench()
+    t = b.measured_traffic_c3()
+    assert set(t) >= {"bs_attention_kernel", "bias_residual_layernorm_kernel", "bias_gelu_kernel", "qkv_bias_split_kernel"}
+    tokens, hidden, ffn = 37184, 768, 3072
+    assert abs(t["bias_residual_layernorm_kernel"] / (3 * tokens * hidden * 2) - 1) < 0.01
+    assert abs(t["bias_gelu_kernel"] / (2 * tokens * ffn * 2) - 1) < 0.01
+    assert abs(t["qkv_bias_split_kernel"] / (2 * tokens * 2 * hidden * 2) - 1) < 0.01
+    assert 4 * tokens * hidden * 2 <= t["bs_attention_kernel"] <= 3 * 4 * tokens * hidden * 2
