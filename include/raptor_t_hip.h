@@ -315,7 +315,8 @@ int rt_pooler_dense_tanh(const void* pooled, const void* weight_t, const void* b
  * layers/multi_headed_attention.h:102-103, .cpp:16-139).  One worker thread per layer
  * waits on a counting semaphore; rt_pipeline_publish stores the batch geometry and
  * signals every layer; each worker builds its layer's CSR (seed = layer index) into
- * pinned memory, copies it on a private copy stream and records an event;
+ * pinned memory, uploads it on a private stream (a small kernel that reads the pinned
+ * buffer: a copy call would make the worker wait for the device) and records an event;
  * rt_pipeline_acquire blocks the host until that layer's CSR is queued, then makes the
  * caller's stream wait on the event.  device < 0 keeps everything on the host (the
  * returned pointers are host pointers) so the ordering logic can be exercised without

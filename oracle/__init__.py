@@ -13,14 +13,14 @@ it follows.  What pins each function:
   plans.rand_attn_max_plan, plans.rand_attn_with_head,
   plans.single_block_row_attention, plans.rand_attn_plan
         golden vectors written by the installed HuggingFace `transformers`
-        BigBird code (tests/golden/hf_plan_*.json) plus structural invariants.
+        BigBird code (tests/golden/hf_plans.json) plus structural invariants.
   metadata.to_index_from_rand_attn, metadata.reference_to_index
         layers/test.cpp golden CSR (n=64), closed form sum(10n-18), legality.
   metadata.lpt_partition, metadata.data_metainfo
         layers/test.cpp golden plan (160 CTAs, 12 heads) -- bit exact.
   attention.bigbird_5part
         golden output of the installed HuggingFace BigBird block-sparse
-        attention (tests/golden/hf_attention_*.npz) and the brute force below.
+        attention (tests/golden/hf_attention.npz) and the brute force below.
   attention.multiset_attention
         textbook softmax in fp64 with a log(count) multiplicity mask; special
         cases that reduce to torch SDPA.
