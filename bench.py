@@ -410,8 +410,8 @@ def run_attention_only(args):
         fn = lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads)
     us = time_kernel(fn, args.steps, args.warmup)
     assert bool(torch.isfinite(out).all()), "the attention output is not finite"
-    # the same batch with every sequence 17 tokens short of its last block (a padded serving batch): the kernel then
-    # masks the padded keys, and every unit runs the moving-maximum loop instead of the pipelined one
+    # the same batch with every sequence 17 tokens short of its last block (a padded serving batch): the kernel's second
+    # instantiation, whose pipelined loop takes each row's padded tile last and masks its padded keys there
     tok_d = torch.tensor([n - 17 for n in lens], dtype=torch.int32).cuda()
     masked_us = time_kernel(lambda: capi.bs_attention_fwd(q, k, vt, out, sb_d, heads, idx_d, pos_d, heads, None, None, tok_d),
                             args.steps, args.warmup)
@@ -426,7 +426,7 @@ def run_attention_only(args):
                          "unit": "TFLOP/s", "frac": ach / 2.5e15, "traffic": None},
             "padded_batch": {"us_per_launch": masked_us, "frac": pairs * PAIR_FLOP / (masked_us * 1e-6) / 2.5e15,
                              "how": "every sequence 17 tokens short of its last block (rt_bs_attention_fwd_masked): "
-                                    "padded keys masked, all units on the moving-maximum loop"}}
+                                    "the pipelined loop runs each row's padded tile last and masks its padded keys there"}}
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline_attention()
     return res

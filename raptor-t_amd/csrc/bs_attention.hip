@@ -554,12 +554,56 @@ __device__ inline void request_first(const Buffers<T>& b, int so, int lane, Tile
     for (int e = 0; e < 8; ++e) t.vf[(f & 1) + 2 + 4 * (f >> 1)][e] = static_cast<T>(0.f);
 }
 
+// Padding of a sequence's last block, for the pipelined loop (MASKED kernels).  pad_off = byte offset (inside K /
+// V^T) of the tile whose keys from `tail` on are padding, -1 if the sequence has none.  The loop masks in its last
+// tile only, so a row's padded tile is moved to the end of the wave's tile list first (the order of a row's tiles
+// does not matter to the result beyond rounding; the reference comes from the first tile).  Key of accumulator
+// element e, key half kt, for this lane: 32 kt + 8 (e >> 2) + (e & 3) + 4 (lane >> 5); it is padding if that is
+// >= tail, i.e. if the part that does not depend on the lane is >= lim.
+struct Padding { int pad_off, lim; bool last; };
+__device__ inline Padding padding_of(const Unit& u, int goff, int lane) {
+  Padding pd;
+  pd.pad_off = u.tail < 64 ? goff + (u.n - 1) * 8192 : -1;
+  pd.lim = u.tail - 4 * (lane >> 5);
+  pd.last = false;
+  return pd;
+}
+// Lanes 0 .. my-1 of ids hold the tile offsets of the wave's entries.  Moves the padded tile to lane my-1 and sets
+// pd.last.  False: the pipelined loop cannot run this list (the padded tile is listed more than once, or it is the
+// first of several, which a hand-over from the previous row may already have requested as the first tile).
+__device__ inline bool pad_to_end(int& ids, int my, int lane, Padding& pd) {
+  pd.last = false;
+  if (pd.pad_off < 0) return true;
+  const unsigned long long m = __ballot(lane < my && ids == pd.pad_off);
+  if (m == 0) return true;
+  if (__popcll(m) > 1) return false;
+  const int jp = __builtin_ctzll(m);
+  if (jp == 0 && my > 1) return false;
+  if (jp != my - 1) {
+    const int moved = __builtin_amdgcn_readlane(ids, my - 1);
+    ids = lane == jp ? moved : (lane == my - 1 ? pd.pad_off : ids);
+  }
+  pd.last = true;
+  return true;
+}
+// scores of padded keys become minus infinity: no weight
+__device__ inline void mask_padded(f32x16& s, int kt, int lim) {
+  asm volatile("" : "+v"(lim));       // the 16 comparisons are made here, not once per kernel and kept in 32 scalar pairs
+#pragma unroll
+  for (int e = 0; e < 16; ++e) s[e] = (32 * kt + 8 * (e >> 2) + (e & 3) >= lim) ? -INFINITY : s[e];
+}
+
 // reference of the pipelined loop: maximum over the row's first 32 keys, shared by the lane's two
-// queries.  False if the two queries' maxima lie too far apart.
-template <typename T>
-__device__ inline bool fast_reference(const Tiles<T>& t, float& mref) {
+// queries.  False if the two queries' maxima lie too far apart.  pad_first (MASKED only): the row's first tile
+// is the padded one, so keys from the tail on do not count (there is always at least one that does).
+template <typename T, bool MASKED>
+__device__ inline bool fast_reference(const Tiles<T>& t, float& mref, bool pad_first, int lim) {
   typedef Mma<T> P;
   f32x16 s0 = {}, s1 = {};
+  if (MASKED && pad_first) {
+    mask_padded(s0, 0, lim);
+    s1 = s0;
+  }
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     s0 = P::run(t.kf[c], t.qf[0][c], s0);
@@ -580,9 +624,9 @@ __device__ inline bool fast_reference(const Tiles<T>& t, float& mref) {
 // fragment k of the next row's queries into t.qf; called in the last tile's last two steps, once
 // the score products have read the fragment it replaces.
 struct NoNextQ { __device__ void operator()(int) const {} };
-template <typename T, typename NextQ>
+template <typename T, bool MASKED, typename NextQ>
 __device__ inline void fast_loop(const Buffers<T>& b, int ids, int my, const int& so_after, int lane, float mref,
-                                 Tiles<T>& t, State& st, NextQ next_q) {
+                                 Tiles<T>& t, State& st, NextQ next_q, const Padding& pd) {
   typedef typename Mma<T>::v8 v8;
   typedef Mma<T> P;
   state_init(st);
@@ -630,6 +674,8 @@ __device__ inline void fast_loop(const Buffers<T>& b, int ids, int my, const int
       uint32_t w[8];
       uint32_t t01 = 0, t23 = 0, t45 = 0, t67 = 0;
       float lacc = 0.f;
+      // a row's padded tile is its last one (pad_to_end): its scores lose the padded keys before they are exponentiated
+      if (MASKED && LAST && pd.last) mask_padded(cur, S >> 1, pd.lim);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         SB();
@@ -714,7 +760,7 @@ __device__ inline void slow_row(const Args<T>& a, const Buffers<T>& b, const QSi
 // Entries first, first + step, ... of row r through the state with the pipelined loop, no hand-over
 // from or to another row.  False: the row has to be run with the moving-maximum loop instead (more
 // than 64 entries for this wave, or scores that outgrew the reference); the state is then undefined.
-template <typename T>
+template <typename T, bool MASKED>
 __device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const QSide<T>& qbias, const Row& r, int first, int step,
                                 int lane, State& st) {
   Tiles<T> t;
@@ -723,13 +769,15 @@ __device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const QSi
   const int my = __builtin_amdgcn_readfirstlane((r.cnt - first + step - 1) / step);     // this wave's entries
   if (my <= 0) return true;
   if (my > 64) return false;
-  const int ids = row_offsets<T>(a, r, first, step, lane);
+  int ids = row_offsets<T>(a, r, first, step, lane);
+  Padding pd = padding_of(r.u, r.goff, lane);
+  if (MASKED && !pad_to_end(ids, my, lane, pd)) return false;
   request_q<T>(a, b, r.u, lane, t.qf);
   request_first<T>(b, __builtin_amdgcn_readlane(ids, 0), lane, t);
   finish_q<T>(a, qbias, r.u, lane, t.qf);
   float mref;
-  if (!fast_reference<T>(t, mref)) return false;
-  fast_loop<T>(b, ids, my, -1, lane, mref, t, st, NoNextQ{});
+  if (!fast_reference<T, MASKED>(t, mref, pd.last && my == 1, pd.lim)) return false;
+  fast_loop<T, MASKED>(b, ids, my, -1, lane, mref, t, st, NoNextQ{}, pd);
   return sums_finite(st);
 }
 
@@ -758,7 +806,7 @@ __device__ inline bool run_solo(const Args<T>& a, const Buffers<T>& b, const QSi
   const Row r = describe<T>(a, u);
   State st;
   if (FAST) {
-    if (!fast_row<T>(a, b, qbias, r, 0, 1, lane, st)) return false;
+    if (!fast_row<T, MASKED>(a, b, qbias, r, 0, 1, lane, st)) return false;
   } else {
     typename Mma<T>::v8 qf[2][4];
     slow_row<T, MASKED>(a, b, qbias, r, 0, 1, lane, false, qf, st);
@@ -775,7 +823,7 @@ __device__ inline bool run_split4(const Args<T>& a, const Buffers<T>& b, const Q
   const Row r = describe<T>(a, u);
   State st;
   if (FAST) {
-    const bool ok = fast_row<T>(a, b, qbias, r, wave, 4, lane, st);
+    const bool ok = fast_row<T, MASKED>(a, b, qbias, r, wave, 4, lane, st);
     if (__syncthreads_or(!ok)) return false;          // also: the park is free (previous item is over)
   } else {
     typename Mma<T>::v8 qf[2][4];
@@ -973,7 +1021,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
         const Unit first = unit_of_flat(ids4[0]);
         const bool tracked = p - begin < REDO_ENTRIES;         // entries past the flags take the moving-maximum loop
         if (is_global_row(first)) {
-          const bool todo = FAST ? (!MASKED && tracked) : (MASKED || !tracked || s_redo[p - begin] != 0);
+          const bool todo = FAST ? tracked : (!tracked || s_redo[p - begin] != 0);
           if (todo) {
             const bool ok = run_split4<T, MASKED, FAST>(a, b, qbias, first, lane, wave, park);
             if (FAST && threadIdx.x == 0) s_redo[p - begin] = ok ? 0 : 1;
@@ -986,7 +1034,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
         if (wave < run) {
           const int e = p + wave - begin;
           const bool trk = e < REDO_ENTRIES;
-          const bool todo = FAST ? (!MASKED && trk) : (MASKED || !trk || s_redo[e] != 0);
+          const bool todo = FAST ? trk : (!trk || s_redo[e] != 0);
           if (todo) {
             const bool ok = run_solo<T, MASKED, FAST>(a, b, qbias, unit_of_flat(mine_id), lane);
             if (FAST && lane == 0) s_redo[e] = ok ? 0 : 1;
@@ -1045,8 +1093,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           __syncthreads();
           if (item >= n_glob) { drained = true; break; }
         }
-        bool ok = false;
-        if (!MASKED) ok = run_split4<T, MASKED, true>(a, b, qbias, unit_of_row(item), lane, wave, park);
+        const bool ok = run_split4<T, MASKED, true>(a, b, qbias, unit_of_row(item), lane, wave, park);
         if (!ok) {
           if (threadIdx.x == 0) redo_rows[n_rows_redo] = item;
           ++n_rows_redo;
@@ -1118,15 +1165,17 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           Row nx = cur;
           if (has_next) describe_bounds<T>(a, unit_of(item_nx), nx);        // scalar loads, waited for below
           State st;
-          bool ok = !MASKED && cur_short;
+          bool ok = cur_short;
+          float mref = 0.f;
+          Padding pd = padding_of(cur.u, cur.goff, lane);
+          if (MASKED && ok) ok = pad_to_end(ids, cur.cnt, lane, pd);
           if (ok && !primed) {
             request_q<T>(a, b, cur.u, lane, t.qf);
             request_first<T>(b, cur.first_off, lane, t);
           }
-          float mref = 0.f;
           if (ok) {
             finish_q<T>(a, qbias, cur.u, lane, t.qf);
-            ok = fast_reference<T>(t, mref);
+            ok = fast_reference<T, MASKED>(t, mref, pd.last && cur.cnt == 1, pd.lim);
           }
           // the next row's block ids: requested here, looked at in the loop's last tile
           bool nx_short = false;
@@ -1144,8 +1193,8 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           primed = false;
           if (ok) {
             const QPlan qn = q_plan<T>(a, nx.u, lane);      // without a next unit: this unit's queries again
-            fast_loop<T>(b, ids, cur.cnt, nx.first_off, lane, mref, t, st,
-                         [&](int k) { t.qf[k >> 2][k & 3] = fetch_q<T>(b, qn, k); });
+            fast_loop<T, MASKED>(b, ids, cur.cnt, nx.first_off, lane, mref, t, st,
+                                 [&](int k) { t.qf[k >> 2][k & 3] = fetch_q<T>(b, qn, k); }, pd);
             lane = lane_id;
             asm volatile("" : "+v"(lane));
             // The unit after the next one: its ticket is drawn here, behind the tile loop, and looked at once this
