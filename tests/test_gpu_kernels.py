@@ -423,15 +423,20 @@ def test_attention_config2_full_size_properties(capi):
                            np.array(one_idx), np.array(one_pos), 1, scale=1.0 / lh.LOG2E)
     assert (out[sel, h * 64:(h + 1) * 64].float().cpu() - ref).abs().max().item() <= 2e-2
 
-@pytest.mark.parametrize("dtype,n_wg", [(torch.float16, 0), (torch.bfloat16, 0), (torch.float16, 96)])
-def test_attention_padded_tail_matches_oracle(capi, dtype, n_wg):
+@pytest.mark.parametrize("dtype,n_wg,reference_plan", [(torch.float16, 0, False), (torch.bfloat16, 0, False),
+                                                       (torch.float16, 96, False), (torch.float16, 0, True),
+                                                       (torch.bfloat16, 96, True)])
+def test_attention_padded_tail_matches_oracle(capi, dtype, n_wg, reference_plan):
     """Sequences whose last block ends in padding: the keys past the true length get no weight.  Covers a
-    sparse sequence, a full-attention one (below 12 blocks), a tail of a single token, and no padding at all;
-    the padded rows hold large values so that a missed mask shows."""
-    say("attention padded", dtype, n_wg)
+    sparse sequence, a full-attention one (below 12 blocks), a tail of a single token, no padding at all, a
+    sequence of one block (its only tile is the padded one: the pipelined loop's reference has to leave the
+    padded keys out too) and one of two; 768 tokens are 12 blocks, where rows list the last block twice (those
+    take the moving-maximum loop), and the reference's head-shared plan keeps more duplicates still.  The padded
+    rows hold large values so that a missed mask shows."""
+    say("attention padded", dtype, n_wg, reference_plan)
     heads = 4
-    seq_lens = [1024, 320, 832, 768]
-    seq_tokens = [1000, 257, 832, 705]
+    seq_lens = [1024, 320, 832, 768, 64, 128]
+    seq_tokens = [1000, 257, 832, 705, 40, 100]
     t = sum(seq_lens)
     g = torch.Generator().manual_seed(11)
     q, k, v = (torch.randn(t, heads, 64, generator=g) for _ in range(3))
@@ -441,7 +446,8 @@ def test_attention_padded_tail_matches_oracle(capi, dtype, n_wg):
         v[start + real:start + n] = 50.0
         start += n
     q, k, v = (x.to(dtype).cuda() for x in (q, k, v))
-    out, ref = lh.run_attention(capi, q, k, v, seq_lens, heads, seed=2, n_wg=n_wg, seq_tokens=seq_tokens)
+    out, ref = lh.run_attention(capi, q, k, v, seq_lens, heads, seed=2, n_wg=n_wg, seq_tokens=seq_tokens,
+                                mode=capi.RT_PLAN_REFERENCE if reference_plan else None)
     start = 0
     for n, real in zip(seq_lens, seq_tokens):              # real query rows only
         over = lh.excess(out[start:start + real], ref[start:start + real], dtype, k=1.0)
