@@ -147,6 +147,15 @@ __device__ inline void state_init(State& st) {
   st.l[0] = st.l[1] = 0.f;
 }
 
+// Scores of padded keys become minus infinity: no weight.  s = 32 x 32 accumulator tile of key half kt; the key of
+// element e in this lane is 32 kt + 8 (e >> 2) + (e & 3) + 4 (lane >> 5), padding from `tail` on.
+__device__ inline void mask_padded(f32x16& s, int kt, int tail, int lane) {
+  int lim = tail - 4 * (lane >> 5);
+  asm volatile("" : "+v"(lim));       // the 16 comparisons are made here, not once per kernel and kept in 32 scalar pairs
+#pragma unroll
+  for (int e = 0; e < 16; ++e) s[e] = (32 * kt + 8 * (e >> 2) + (e & 3) >= lim) ? -INFINITY : s[e];
+}
+
 template <typename T>
 __device__ inline void load_tile(const T* __restrict__ tile, int lane, typename Mma<T>::v8 (&f)[8]) {
   typedef typename Mma<T>::v8 v8;
@@ -201,11 +210,8 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
           for (int c = 0; c < 4; ++c) sc[t] = Mma<T>::run(kf[t * 4 + c], qf[nt][c], sc[t]);
         }
         if (MASKED && padded) {                         // wave-uniform, at most one tile of a row
-#pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-              if (32 * t + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3) >= tail) sc[t][e] = -INFINITY;
+          mask_padded(sc[0], 0, tail, lane);
+          mask_padded(sc[1], 1, tail, lane);
         }
       };
       // exp2 of the (already shifted) scores -> P as the B operand of the second product:
@@ -559,12 +565,12 @@ __device__ inline void request_first(const Buffers<T>& b, int so, int lane, Tile
 // tile only, so a row's padded tile is moved to the end of the wave's tile list first (the order of a row's tiles
 // does not matter to the result beyond rounding; the reference comes from the first tile).  Key of accumulator
 // element e, key half kt, for this lane: 32 kt + 8 (e >> 2) + (e & 3) + 4 (lane >> 5); it is padding if that is
-// >= tail, i.e. if the part that does not depend on the lane is >= lim.
-struct Padding { int pad_off, lim; bool last; };
-__device__ inline Padding padding_of(const Unit& u, int goff, int lane) {
+// >= tail.
+struct Padding { int pad_off, tail; bool last; };
+__device__ inline Padding padding_of(const Unit& u, int goff) {
   Padding pd;
   pd.pad_off = u.tail < 64 ? goff + (u.n - 1) * 8192 : -1;
-  pd.lim = u.tail - 4 * (lane >> 5);
+  pd.tail = u.tail;
   pd.last = false;
   return pd;
 }
@@ -586,22 +592,16 @@ __device__ inline bool pad_to_end(int& ids, int my, int lane, Padding& pd) {
   pd.last = true;
   return true;
 }
-// scores of padded keys become minus infinity: no weight
-__device__ inline void mask_padded(f32x16& s, int kt, int lim) {
-  asm volatile("" : "+v"(lim));       // the 16 comparisons are made here, not once per kernel and kept in 32 scalar pairs
-#pragma unroll
-  for (int e = 0; e < 16; ++e) s[e] = (32 * kt + 8 * (e >> 2) + (e & 3) >= lim) ? -INFINITY : s[e];
-}
 
 // reference of the pipelined loop: maximum over the row's first 32 keys, shared by the lane's two
 // queries.  False if the two queries' maxima lie too far apart.  pad_first (MASKED only): the row's first tile
 // is the padded one, so keys from the tail on do not count (there is always at least one that does).
 template <typename T, bool MASKED>
-__device__ inline bool fast_reference(const Tiles<T>& t, float& mref, bool pad_first, int lim) {
+__device__ inline bool fast_reference(const Tiles<T>& t, float& mref, bool pad_first, int tail, int lane) {
   typedef Mma<T> P;
   f32x16 s0 = {}, s1 = {};
   if (MASKED && pad_first) {
-    mask_padded(s0, 0, lim);
+    mask_padded(s0, 0, tail, lane);
     s1 = s0;
   }
 #pragma unroll
@@ -675,7 +675,7 @@ __device__ inline void fast_loop(const Buffers<T>& b, int ids, int my, const int
       uint32_t t01 = 0, t23 = 0, t45 = 0, t67 = 0;
       float lacc = 0.f;
       // a row's padded tile is its last one (pad_to_end): its scores lose the padded keys before they are exponentiated
-      if (MASKED && LAST && pd.last) mask_padded(cur, S >> 1, pd.lim);
+      if (MASKED && LAST && pd.last) mask_padded(cur, S >> 1, pd.tail, lane);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         SB();
@@ -770,13 +770,13 @@ __device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const QSi
   if (my <= 0) return true;
   if (my > 64) return false;
   int ids = row_offsets<T>(a, r, first, step, lane);
-  Padding pd = padding_of(r.u, r.goff, lane);
+  Padding pd = padding_of(r.u, r.goff);
   if (MASKED && !pad_to_end(ids, my, lane, pd)) return false;
   request_q<T>(a, b, r.u, lane, t.qf);
   request_first<T>(b, __builtin_amdgcn_readlane(ids, 0), lane, t);
   finish_q<T>(a, qbias, r.u, lane, t.qf);
   float mref;
-  if (!fast_reference<T, MASKED>(t, mref, pd.last && my == 1, pd.lim)) return false;
+  if (!fast_reference<T, MASKED>(t, mref, pd.last && my == 1, pd.tail, lane)) return false;
   fast_loop<T, MASKED>(b, ids, my, -1, lane, mref, t, st, NoNextQ{}, pd);
   return sums_finite(st);
 }
@@ -1167,7 +1167,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           State st;
           bool ok = cur_short;
           float mref = 0.f;
-          Padding pd = padding_of(cur.u, cur.goff, lane);
+          Padding pd = padding_of(cur.u, cur.goff);
           if (MASKED && ok) ok = pad_to_end(ids, cur.cnt, lane, pd);
           if (ok && !primed) {
             request_q<T>(a, b, cur.u, lane, t.qf);
@@ -1175,7 +1175,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           }
           if (ok) {
             finish_q<T>(a, qbias, cur.u, lane, t.qf);
-            ok = fast_reference<T, MASKED>(t, mref, pd.last && cur.cnt == 1, pd.lim);
+            ok = fast_reference<T, MASKED>(t, mref, pd.last && cur.cnt == 1, pd.tail, lane);
           }
           // the next row's block ids: requested here, looked at in the loop's last tile
           bool nx_short = false;
