@@ -187,9 +187,11 @@ int rt_bs_attention_fwd(const void* q, const void* k, const void* vt, void* out,
 /* The same launch for a batch whose sequences end in padding (the reference only takes
  * lengths that are multiples of 64: python/util.py:36-46; this is the to_mask / band_mask /
  * rand_mask handling of its oracle, python/modeling_big_bird.py:640-760, for a packed batch).
- * seq_tokens_dev[s] = true token count of sequence s, in (64 * (n_s - 1), 64 * n_s]; the keys from
- * there to the end of the sequence's last block get no weight.  Padded QUERY rows are computed
- * like any other row; the caller drops them.  NULL = no padding (rt_bs_attention_fwd). */
+ * seq_tokens_dev[s] = true token count of sequence s, 1 .. 64 * n_s (values outside are clamped); the
+ * keys from there to the end of the sequence get no weight, whether they are the tail of one block or
+ * whole blocks (a sequence kept at the width of a padded batch, so that its plan is the one the oracle
+ * draws for that width).  Padded QUERY rows are computed like any other row (over the real keys their
+ * rows list); the caller drops them.  NULL = no padding (rt_bs_attention_fwd). */
 int rt_bs_attention_fwd_masked(const void* q, const void* k, const void* vt, void* out,
                                const int* seq_blocks_dev, const int* seq_tokens_dev, int batch,
                                int total_blocks, int heads, const int* to_idx, const int* to_pos,

@@ -169,7 +169,7 @@ __device__ inline void load_tile(const T* __restrict__ tile, int lane, typename 
 // entry j) and handed out with v_readlane: one memory round trip per unit instead of one per key block.
 template <typename T, bool MASKED>
 __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __restrict__ vbase,
-                                    const int* __restrict__ row, int first, int step, int cnt, int n, int tail,
+                                    const int* __restrict__ row, int first, int step, int cnt, int n, int tail, int nbv,
                                     int lane, const typename Mma<T>::v8 (&qf)[2][4], State& st) {
   typedef typename Mma<T>::v8 v8;
   v8 kf[8], vf[8];
@@ -191,8 +191,10 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
   for (; j < hi; j += step) {
     const int jn = j + step;
     const bool more = jn < hi;
-    // keys of the sequence's last block beyond its true length are padding: no weight
-    const bool padded = MASKED && tail < 64 && bcur == n - 1;
+    // keys beyond the sequence's true length are padding and get no weight: the tail of block nbv - 1 is masked, a
+    // block from nbv on is left out as a whole (its tile has been requested like any other and is dropped)
+    const bool padded = MASKED && tail < 64 && bcur == nbv - 1;
+    const bool skipped = MASKED && bcur >= nbv;
     // the last iteration re-requests its own tile: loads stay unconditional, so they keep
     // their place in the instruction stream (a branch would sink them next to their use)
     const int bn = block_of(more ? jn : j);
@@ -229,8 +231,8 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
         psum = (part[0] + part[1]) + (part[2] + part[3]);
         return !(psum <= SUM_LIMIT);                    // also true for an infinite or undefined sum
       };
-      bool redo = fresh;
-      if (!fresh) {
+      bool redo = fresh && !skipped;
+      if (!fresh && !skipped) {
         scores(-st.m[nt]);
         redo = __any(exponentiate());
       }
@@ -265,13 +267,15 @@ __device__ inline void stream_tiles(const T* __restrict__ kbase, const T* __rest
         load_tile<T>(kbase + int64_t(bn) * 4096, lane, kf);
         __builtin_amdgcn_sched_barrier(0);
       }
-      st.l[nt] += psum;
+      if (!skipped) {
+        st.l[nt] += psum;
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int s = 0; s < 4; ++s) st.o[t][nt] = Mma<T>::run(vf[t * 4 + s], pb[s], st.o[t][nt]);
+          for (int s = 0; s < 4; ++s) st.o[t][nt] = Mma<T>::run(vf[t * 4 + s], pb[s], st.o[t][nt]);
+      }
     }
-    fresh = false;
+    fresh = fresh && skipped;
     bcur = bn;
     __builtin_amdgcn_sched_barrier(0);
     load_tile<T>(vbase + int64_t(bn) * 4096, lane, vf);
@@ -334,7 +338,9 @@ __device__ inline void store_output(T* __restrict__ out_unit, int64_t row_stride
 
 struct Unit {
   int h, i, n, g0;
-  int tail;               // tokens in the sequence's last block that are real (64: none padded)
+  int tail;               // real tokens in the sequence's last block that holds any (64: none padded)
+  int nbv;                // blocks of the sequence that hold real tokens (n without padding): blocks from nbv on are
+                          // padding as a whole and get no weight as keys
 };
 
 // One unit's row of the to-block CSR, for the wave that runs it (all fields wave-uniform).
@@ -376,7 +382,8 @@ struct Geometry {
   int sb[MAX_BATCH + 1];                // prefix blocks
   uint32_t rows[MAX_BLOCKS];            // j-th row that is not a global row: sequence << 16 | block inside the sequence
   uint16_t sparse_seq[MAX_BATCH];       // k-th sequence that has global rows
-  uint8_t tail[MAX_BATCH];              // real tokens in each sequence's last block (64 without padding)
+  uint8_t tail[MAX_BATCH];              // real tokens in each sequence's last block that holds any (64 without padding)
+  uint16_t nbv[MAX_BATCH];              // blocks of each sequence that hold real tokens
   int n_rows, n_sparse;
 };
 
@@ -560,25 +567,38 @@ __device__ inline void request_first(const Buffers<T>& b, int so, int lane, Tile
     for (int e = 0; e < 8; ++e) t.vf[(f & 1) + 2 + 4 * (f >> 1)][e] = static_cast<T>(0.f);
 }
 
-// Padding of a sequence's last block, for the pipelined loop (MASKED kernels).  pad_off = byte offset (inside K /
-// V^T) of the tile whose keys from `tail` on are padding, -1 if the sequence has none.  The loop masks in its last
-// tile only, so a row's padded tile is moved to the end of the wave's tile list first (the order of a row's tiles
-// does not matter to the result beyond rounding; the reference comes from the first tile).  Key of accumulator
-// element e, key half kt, for this lane: 32 kt + 8 (e >> 2) + (e & 3) + 4 (lane >> 5); it is padding if that is
-// >= tail.
-struct Padding { int pad_off, tail; bool last; };
+// Padding of a sequence, for the pipelined loop (MASKED kernels).  drop_off = byte offset (inside K / V^T) of the
+// sequence's first block that is padding as a whole: tiles from there on are taken off the wave's tile list.
+// pad_off = offset of the tile whose keys from `tail` on are padding, -1 if there is none.  The loop masks in its
+// last tile only, so a row's padded tile is moved to the end of the list (the order of a row's tiles does not matter
+// to the result beyond rounding; the reference comes from the first tile).
+struct Padding { int pad_off, drop_off, tail; bool last; };
 __device__ inline Padding padding_of(const Unit& u, int goff) {
   Padding pd;
-  pd.pad_off = u.tail < 64 ? goff + (u.n - 1) * 8192 : -1;
+  pd.pad_off = u.tail < 64 ? goff + (u.nbv - 1) * 8192 : -1;
+  pd.drop_off = goff + u.nbv * 8192;
   pd.tail = u.tail;
   pd.last = false;
   return pd;
 }
-// Lanes 0 .. my-1 of ids hold the tile offsets of the wave's entries.  Moves the padded tile to lane my-1 and sets
-// pd.last.  False: the pipelined loop cannot run this list (the padded tile is listed more than once, or it is the
-// first of several, which a hand-over from the previous row may already have requested as the first tile).
-__device__ inline bool pad_to_end(int& ids, int my, int lane, Padding& pd) {
+// Lanes 0 .. my-1 of ids hold the tile offsets of the wave's entries.  Takes the tiles that are padding as a whole
+// off the list (my shrinks), moves the padded tile to the last lane in use and sets pd.last.  False: the pipelined
+// loop cannot run this list (the padded tile is listed more than once, or the list's first tile does not stay
+// first, which a hand-over from the previous row may already have requested).
+__device__ inline bool pad_to_end(int& ids, int& my, int lane, Padding& pd) {
   pd.last = false;
+  const unsigned long long listed = __ballot(lane < my);
+  const unsigned long long keep = __ballot(lane < my && ids < pd.drop_off);
+  if (keep != listed) {
+    if (!(keep & 1ull)) return false;
+    // kept entries move up in order; the dropped ones go behind them, lanes beyond the list stay (a permutation)
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const int kept = __popcll(keep);
+    const bool mine = (keep >> lane) & 1ull;
+    const int dest = lane >= my ? lane : (mine ? __popcll(keep & below) : kept + __popcll(listed & ~keep & below));
+    ids = __builtin_amdgcn_ds_permute(dest * 4, ids);
+    my = kept;
+  }
   if (pd.pad_off < 0) return true;
   const unsigned long long m = __ballot(lane < my && ids == pd.pad_off);
   if (m == 0) return true;
@@ -754,7 +774,7 @@ __device__ inline void slow_row(const Args<T>& a, const Buffers<T>& b, const QSi
   }
   state_init(st);
   const int64_t gbase = int64_t(r.goff >> 1);
-  stream_tiles<T, MASKED>(a.k + gbase, a.vt + gbase, a.to_idx + r.p0, first, step, r.cnt, r.u.n, r.u.tail, lane, qf, st);
+  stream_tiles<T, MASKED>(a.k + gbase, a.vt + gbase, a.to_idx + r.p0, first, step, r.cnt, r.u.n, r.u.tail, r.u.nbv, lane, qf, st);
 }
 
 // Entries first, first + step, ... of row r through the state with the pipelined loop, no hand-over
@@ -766,12 +786,15 @@ __device__ inline bool fast_row(const Args<T>& a, const Buffers<T>& b, const QSi
   Tiles<T> t;
   state_init(st);
   first = __builtin_amdgcn_readfirstlane(first);
-  const int my = __builtin_amdgcn_readfirstlane((r.cnt - first + step - 1) / step);     // this wave's entries
+  int my = __builtin_amdgcn_readfirstlane((r.cnt - first + step - 1) / step);           // this wave's entries
   if (my <= 0) return true;
   if (my > 64) return false;
   int ids = row_offsets<T>(a, r, first, step, lane);
   Padding pd = padding_of(r.u, r.goff);
-  if (MASKED && !pad_to_end(ids, my, lane, pd)) return false;
+  if (MASKED) {
+    if (!pad_to_end(ids, my, lane, pd)) return false;
+    if (my == 0) return true;                          // every tile of this wave's share is padding
+  }
   request_q<T>(a, b, r.u, lane, t.qf);
   request_first<T>(b, __builtin_amdgcn_readlane(ids, 0), lane, t);
   finish_q<T>(a, qbias, r.u, lane, t.qf);
@@ -932,11 +955,14 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       before_in_wave[r] = __popcll(votes & ((1ull << lane) - 1ull));
       if (lane == 0) wave_sparse[r * 4 + wave] = __popcll(votes);
       if (sq < a.batch) {
-        int t = 64;
-        if (MASKED) {
-          t = a.seq_tokens[sq] - 64 * (geo.sb[sq + 1] - geo.sb[sq] - 1);
-          t = t < 1 ? 1 : (t > 64 ? 64 : t);
+        const int nblk = geo.sb[sq + 1] - geo.sb[sq];
+        int t = 64, nv = nblk;
+        if (MASKED) {                                                // at least one real token, at most the sequence
+          const int tokens = min(max(a.seq_tokens[sq], 1), 64 * nblk);
+          nv = (tokens + 63) >> 6;
+          t = tokens - 64 * (nv - 1);
         }
+        geo.nbv[sq] = uint16_t(nv);
         geo.tail[sq] = uint8_t(t);
       }
     }
@@ -992,6 +1018,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
     u.g0 = geo.sb[lo];
     u.n = geo.sb[lo + 1] - u.g0;
     u.tail = geo.tail[lo];
+    u.nbv = MASKED ? int(geo.nbv[lo]) : u.n;
     const int rem = unit - u.g0 * a.heads;
     u.h = rem / u.n;
     u.i = rem - u.h * u.n;
@@ -1069,6 +1096,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       u.g0 = geo.sb[s];
       u.n = geo.sb[s + 1] - u.g0;
       u.tail = geo.tail[s];
+      u.nbv = MASKED ? int(geo.nbv[s]) : u.n;
       u.h = h;
       u.i = (ticket & 1) ? u.n - 1 : 0;
       return u;
@@ -1126,6 +1154,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
       u.g0 = geo.sb[s];
       u.n = geo.sb[s + 1] - u.g0;
       u.tail = geo.tail[s];
+      u.nbv = MASKED ? int(geo.nbv[s]) : u.n;
       u.h = h;
       u.i = int(e & 0xffffu);
       return u;
@@ -1168,14 +1197,15 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           bool ok = cur_short;
           float mref = 0.f;
           Padding pd = padding_of(cur.u, cur.goff);
-          if (MASKED && ok) ok = pad_to_end(ids, cur.cnt, lane, pd);
+          int my = cur.cnt;                                 // tiles of the row that the loop runs
+          if (MASKED && ok) ok = pad_to_end(ids, my, lane, pd);
           if (ok && !primed) {
             request_q<T>(a, b, cur.u, lane, t.qf);
             request_first<T>(b, cur.first_off, lane, t);
           }
           if (ok) {
             finish_q<T>(a, qbias, cur.u, lane, t.qf);
-            ok = fast_reference<T, MASKED>(t, mref, pd.last && cur.cnt == 1, pd.tail, lane);
+            ok = fast_reference<T, MASKED>(t, mref, pd.last && my == 1, pd.tail, lane);
           }
           // the next row's block ids: requested here, looked at in the loop's last tile
           bool nx_short = false;
@@ -1193,7 +1223,7 @@ __global__ __launch_bounds__(256, 2) void bs_attention_kernel(Args<T> a) {
           primed = false;
           if (ok) {
             const QPlan qn = q_plan<T>(a, nx.u, lane);      // without a next unit: this unit's queries again
-            fast_loop<T, MASKED>(b, ids, cur.cnt, nx.first_off, lane, mref, t, st,
+            fast_loop<T, MASKED>(b, ids, my, nx.first_off, lane, mref, t, st,
                                  [&](int k) { t.qf[k >> 2][k & 3] = fetch_q<T>(b, qn, k); }, pd);
             lane = lane_id;
             asm volatile("" : "+v"(lane));

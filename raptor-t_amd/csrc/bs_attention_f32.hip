@@ -88,8 +88,10 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
   const int g0 = a.seq_blocks[lo], n = a.seq_blocks[lo + 1] - g0;
   const int rem = unit - g0 * a.heads;
   const int h = rem / n, i = rem - h * n;
-  // real tokens of the last block; at least one (a tile with every key masked has no finite maximum)
-  const int tail = MASKED ? min(max(a.seq_tokens[lo] - 64 * (n - 1), 1), 64) : 64;
+  // blocks that hold real tokens and the real tokens of the last of them; at least one (a tile with every key
+  // masked has no finite maximum); blocks from nbv on are padding as a whole and are left out
+  const int tokens = MASKED ? min(max(a.seq_tokens[lo], 1), 64 * n) : 64 * n;
+  const int nbv = (tokens + 63) >> 6, tail = tokens - 64 * (nbv - 1);
   const int row = (a.plan_heads > 1 ? h : 0) * a.nb_total + g0 + i;
   const int p0 = a.to_pos[row], p1 = a.to_pos[row + 1];
   const int64_t head_base = (int64_t(g0) * a.heads + int64_t(h) * n) * 4096;
@@ -122,6 +124,7 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
 
   for (int p = p0; p < p1; ++p) {
     const int blk = min(max(a.to_idx[p], 0), n - 1);   // a malformed index must not lead outside the (sequence, head)
+    if (MASKED && blk >= nbv) continue;                // the same in every thread of the workgroup
     __syncthreads();                                   // the previous tile's readers are done
     stage_tile<false>(a.k + head_base + int64_t(blk) * 4096, ks);
     stage_tile<true>(a.vt + head_base + int64_t(blk) * 4096, vs);
@@ -134,7 +137,7 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
       for (int st = 0; st < 16; ++st)
         s[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ks[16 * kt + qcol][4 * st + grp], qreg[st], s[kt], 0, 0, 0);
     }
-    if (MASKED && blk == n - 1 && tail < 64) {
+    if (MASKED && blk == nbv - 1 && tail < 64) {
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
@@ -170,7 +173,7 @@ __device__ void run_unit(const ArgsF32& a, int unit, float (*ks)[PITCH], float (
     }
   }
   // O^T accumulator dt: lane holds d = 16 dt + 4 grp + e for query qcol
-  const float inv = 1.0f / l;
+  const float inv = 1.0f / fmaxf(l, 1e-30f);          // a row that lists nothing but padding writes zeros
   float* dst = a.out + (int64_t(g0 + i) * 64 + 16 * wave + qcol) * dm + h * 64;
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt) *reinterpret_cast<f32x4*>(dst + 16 * dt + 4 * grp) = o[dt] * inv;

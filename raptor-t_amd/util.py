@@ -83,12 +83,17 @@ def uniform_lengths(batch, lo, hi, seed=0, block=64):
     return (block * rng.integers(lo // block, hi // block + 1, size=batch)).tolist()
 
 
-def pack_padded_batch(input_ids, attention_mask, token_type_ids=None, block_size=64):
+def pack_padded_batch(input_ids, attention_mask, token_type_ids=None, block_size=64, keep_width=False):
     """Padded HuggingFace-style batch -> the packed batch the encoder takes.
 
     input_ids, attention_mask: [B, L] (mask 1 on real tokens, which must be a prefix of each row).  Every
     sequence keeps its real tokens plus the padding needed to fill its own last 64-token block (the
-    reference only takes lengths that are multiples of 64, python/util.py:36-46).  Returns a dict:
+    reference only takes lengths that are multiples of 64, python/util.py:36-46): the cheapest batch, in which
+    every sequence gets the attention plan of its own length.  keep_width=True keeps every sequence at the
+    batch's width L (rounded up to a block) instead, whole blocks of padding included: the plan of every
+    sequence is then the one HuggingFace BigBird draws for the padded batch (python/modeling_big_bird.py:573-597
+    chooses it by the padded length), so the real rows equal HuggingFace run on the padded batch itself, at the
+    price of computing the padding.  Returns a dict:
       input_ids, position_ids, token_type_ids : int32 [T] packed, T = sum(seq_lens)
       seq_lens   : per-sequence packed length, a multiple of block_size
       seq_tokens : per-sequence true token count (list) and `seq_tokens_tensor` (int32, on the ids' device):
@@ -106,6 +111,8 @@ def pack_padded_batch(input_ids, attention_mask, token_type_ids=None, block_size
     if min(seq_tokens) < 1:
         raise ValueError("every sequence needs at least one token")
     seq_lens = [(n + block_size - 1) // block_size * block_size for n in seq_tokens]
+    if keep_width:
+        seq_lens = [(length + block_size - 1) // block_size * block_size] * b
     pad_to = max(seq_lens)
     if pad_to > length:                                   # the padded width is not a block multiple itself
         extra = pad_to - length

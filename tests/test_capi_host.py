@@ -277,6 +277,13 @@ def test_padded_batch_adapters_round_trip():
     assert back.shape == (3, width, 2)
     assert torch.equal(back[0, :130], hidden[:130]) and torch.equal(back[2, 0], hidden[256])
     assert back[0, 130:].abs().sum() == 0 and back[2, 1:].abs().sum() == 0
+    # every sequence kept at the batch's width (rounded up to a block): whole blocks of padding stay
+    w = ut.pack_padded_batch(ids, mask, keep_width=True)
+    assert w["seq_lens"] == [192, 192, 192] and w["seq_tokens"] == lens and w["input_ids"].numel() == 576
+    assert w["input_ids"][192:192 + 150].tolist() == ids[1].tolist() and w["input_ids"][192 + 150:384].abs().sum() == 0
+    assert w["position_ids"][384:576].tolist() == list(range(192))
+    back = ut.unpack_to_padded(torch.arange(576 * 2, dtype=torch.float32).view(576, 2), w["seq_lens"], w["seq_tokens"], width)
+    assert back.shape == (3, width, 2) and back[1, 64:].abs().sum() == 0 and back[1, 63, 0] == 2 * (192 + 63)
     with pytest.raises(ValueError):
         ut.pack_padded_batch(ids, torch.tensor([[1, 0, 1]]).expand(3, 3)[:, :3].repeat(1, 50))   # holes in the mask
     with pytest.raises(ValueError):

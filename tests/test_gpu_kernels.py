@@ -437,6 +437,25 @@ def test_attention_padded_tail_matches_oracle(capi, dtype, n_wg, reference_plan)
     heads = 4
     seq_lens = [1024, 320, 832, 768, 64, 128]
     seq_tokens = [1000, 257, 832, 705, 40, 100]
+    _check_padded_attention(capi, dtype, n_wg, reference_plan, heads, seq_lens, seq_tokens)
+
+
+@pytest.mark.parametrize("dtype,n_wg,reference_plan", [(torch.float16, 0, False), (torch.bfloat16, 0, False),
+                                                       (torch.float32, 0, False), (torch.float16, 96, False),
+                                                       (torch.bfloat16, 0, True)])
+def test_attention_padded_blocks_match_oracle(capi, dtype, n_wg, reference_plan):
+    """Sequences kept at a padded batch's width: whole blocks of padding behind the real tokens.  Their keys get no
+    weight (the tiles are taken off the pipelined loop's list), the block the real tokens end in is masked from
+    the tail on.  Covers real tokens ending inside a block and exactly at a block's end, a single real block, a
+    single real token, and a sequence without padding beside them."""
+    say("attention padded blocks", dtype, n_wg, reference_plan)
+    heads = 4
+    seq_lens = [1024, 1024, 1024, 768, 320, 1024, 832]
+    seq_tokens = [700, 128, 50, 100, 64, 1, 832]
+    _check_padded_attention(capi, dtype, n_wg, reference_plan, heads, seq_lens, seq_tokens)
+
+
+def _check_padded_attention(capi, dtype, n_wg, reference_plan, heads, seq_lens, seq_tokens):
     t = sum(seq_lens)
     g = torch.Generator().manual_seed(11)
     q, k, v = (torch.randn(t, heads, 64, generator=g) for _ in range(3))
@@ -737,7 +756,10 @@ def test_attention_random_geometries(capi):
         mode = capi.RT_PLAN_REFERENCE if rng.integers(0, 4) == 0 else None
         n_wg = int(rng.integers(1, 60)) if rng.integers(0, 2) else 0
         padded = bool(rng.integers(0, 2))
-        seq_tokens = [n - int(rng.integers(0, 64)) for n in lens] if padded else None
+        wide = bool(rng.integers(0, 2))                    # padding of whole blocks, not only of a block's tail
+        seq_tokens = None
+        if padded:
+            seq_tokens = [int(rng.integers(1, n + 1)) if wide else n - int(rng.integers(0, 64)) for n in lens]
         say("  case", case, lens, heads, dtype, mode, n_wg, seq_tokens)
         t = sum(lens)
         g = torch.Generator().manual_seed(1000 + case)

@@ -577,6 +577,52 @@ def test_padded_batch_of_several_sequences_matches_huggingface_per_sequence(mb, 
         assert bool((got[s, real:] == 0).all())
 
 
+def test_padded_batch_kept_at_its_width_matches_huggingface_on_the_padded_batch(mb, ut):
+    """The same kind of batch with every sequence kept at the padded width (pack_padded_batch(keep_width=True)):
+    whole blocks of padding stay in the packed batch, every sequence gets the plan HuggingFace draws for the
+    padded length, and the real rows equal HuggingFace BigBird run ONCE on the padded batch with its attention
+    mask.  Fills: nearly full, ending inside a block in the middle, ending exactly at a block's end, and three
+    blocks of sixteen."""
+    say("hf padded batch, kept width")
+    from transformers import BigBirdConfig, BigBirdModel
+    torch.manual_seed(6)
+    cfg = BigBirdConfig(vocab_size=1000, hidden_size=128, num_hidden_layers=2, num_attention_heads=2,
+                        intermediate_size=256, max_position_embeddings=4096, attention_type="block_sparse",
+                        block_size=64, num_random_blocks=3, hidden_dropout_prob=0.0,
+                        attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+    hf = BigBirdModel(cfg, add_pooling_layer=False).cuda().train()
+    with torch.no_grad():
+        for layer in hf.encoder.layer:
+            layer.attention.self.query.weight.mul_(6.0)
+            layer.attention.self.key.weight.mul_(6.0)
+            layer.attention.self.value.weight.mul_(5.0)
+    length, tokens = 1024, [1000, 700, 832, 130]
+    ids = torch.randint(1, 1000, (len(tokens), length), device="cuda")       # padding ids are not zero: a missed mask shows
+    mask = (torch.arange(length, device="cuda")[None, :] < torch.tensor(tokens, device="cuda")[:, None]).long()
+    with torch.no_grad():
+        want = hf(input_ids=ids, attention_mask=mask).last_hidden_state.float().cpu()
+        unmasked = hf(input_ids=ids).last_hidden_state.float().cpu()
+    assert (want[3, :130] - unmasked[3, :130]).abs().max().item() > 5e-2      # the mask matters for this input
+    p = ut.pack_padded_batch(ids, mask, keep_width=True)
+    assert p["seq_lens"] == [1024] * 4 and p["seq_tokens"] == tokens
+    model = mb.BertModelNoPooler.from_torch(hf, async_=True, dtype=torch.float16)
+    t = sum(p["seq_lens"])
+    meta = mb.cxx.MetaData()
+    spi, spi_t, total_comp, ppi_t, pp_t = ut.generate_data_metainfo(p["seq_lens"], 64, 48, 2)
+    meta.update_meta_data(t, spi[-1] + 1, total_comp, spi)
+    inter = torch.empty(t, 256, dtype=torch.float16, device="cuda")
+    out, _ = model(p["input_ids"], t, 48, spi, spi_t, ppi_t, pp_t, attention_masks=p["seq_tokens_tensor"],
+                   token_type_ids=p["token_type_ids"], position_ids=p["position_ids"], intermediate_temp=inter)
+    torch.cuda.synchronize()
+    meta.terminate_thread()
+    got = ut.unpack_to_padded(out, p["seq_lens"], p["seq_tokens"], length)
+    for s, real in enumerate(tokens):
+        err = (got[s, :real].float().cpu() - want[s, :real]).abs().max().item()
+        say("  sequence", s, "tokens", real, "err", err)
+        assert err <= 2e-2
+        assert bool((got[s, real:] == 0).all())
+
+
 def _run_headline_workload(pkg, mb, ut, name, two_streams, keep_rows=None):
     """bench.py's encoder workload `name` once through the layer API (asynchronous block-index pipeline, the step
     bench.py times).  keep_rows (a slice of token rows, one stream only): the layers are called one by one, as
