@@ -666,6 +666,10 @@ __device__ inline void fast_loop(const Buffers<T>& b, int ids, int my, const int
   // derives them from the state at the loop's entry as well as from the loop's own requests, and
   // anything still pending there turns them into waits for all requests.
   __builtin_amdgcn_s_waitcnt(0x0F70);                 // vmcnt(0)
+  // Inside the loop a wave yields to the other wave of its SIMD whenever that one is between two loops (queries,
+  // reference, output, the next row's description): that code is a chain of short latencies, the loop always has
+  // matrix work in flight.  Worth 2 % where rows are long (8 x 4096 tokens), nothing elsewhere.
+  __builtin_amdgcn_s_setprio(0);
   SB();
   // pipeline prologue: scores of the first accumulator tile; an all-zero P for the first step's PV slot
   sc[0] = negm;
@@ -760,6 +764,7 @@ __device__ inline void fast_loop(const Buffers<T>& b, int ids, int my, const int
     for (int s = 0; s < 2; ++s) st.o[tt][1] = P::run(t.vf[tt * 4 + 2 + s], pb[1][s], st.o[tt][1]);
   st.l[0] = l0;
   st.l[1] = l1;
+  __builtin_amdgcn_s_setprio(1);
 }
 
 __device__ inline bool sums_finite(const State& st) { return !__any(!(st.l[0] < INFINITY) || !(st.l[1] < INFINITY)); }
